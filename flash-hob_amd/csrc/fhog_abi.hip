@@ -1,0 +1,154 @@
+// C ABI of libfhog_hip.so: argument validation, kernel-family selection, pass sequencing.
+// Replaces the host side of flash_bwdbwd (fhog/triton_bwdbwd.py:557-648).
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "fhog_common.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int validate(const fhog_bwdbwd_args* a) {
+  if (!a) return fail(FHOG_E_NULL, "args is NULL");
+  const void* ptrs[] = {a->q, a->k, a->v, a->o, a->dO, a->ddq, a->ddk, a->ddv, a->lse, a->dq2, a->dk2, a->dv2, a->ddo, a->ws};
+  const char* names[] = {"q", "k", "v", "o", "dO", "ddq", "ddk", "ddv", "lse", "dq2", "dk2", "dv2", "ddo", "ws"};
+  for (int i = 0; i < 14; i++)
+    if (!ptrs[i]) return fail(FHOG_E_NULL, "pointer '%s' is NULL", names[i]);
+  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
+  if (a->impl != FHOG_IMPL_AUTO && a->impl != FHOG_IMPL_FP32 && a->impl != FHOG_IMPL_BF16)
+    return fail(FHOG_E_DTYPE, "unknown impl %d", a->impl);
+  if (a->batch < 1 || a->n_q < 1 || a->n_k < 1)
+    return fail(FHOG_E_SHAPE, "batch, n_q, n_k must be >= 1 (got %lld, %lld, %lld)", (long long)a->batch, (long long)a->n_q,
+                (long long)a->n_k);
+  if (a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)a->batch);
+  if (a->n_q > (1 << 24) || a->n_k > (1 << 24)) return fail(FHOG_E_SHAPE, "n_q/n_k above 2^24 not supported");
+  if (a->batch * a->n_q >= (int64_t)1 << 31) return fail(FHOG_E_SHAPE, "batch*n_q must be below 2^31");
+  if (a->d != 32 && a->d != 64 && a->d != 128) return fail(FHOG_E_SHAPE, "head dim %lld not in {32, 64, 128}", (long long)a->d);
+  if (a->causal != 0 && a->causal != 1) return fail(FHOG_E_CAUSAL, "causal must be 0 or 1");
+  if (a->causal && a->n_q != a->n_k)
+    return fail(FHOG_E_CAUSAL, "causal needs n_q == n_k (got %lld, %lld)", (long long)a->n_q, (long long)a->n_k);
+  if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
+  const int vec = a->dtype == FHOG_DTYPE_BF16 ? 8 : 4;  // elements per 16 bytes
+  if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
+  if (a->stride_qn % vec || a->stride_kn % vec || a->stride_qb % vec || a->stride_kb % vec)
+    return fail(FHOG_E_STRIDE, "strides must be multiples of %d elements (16 bytes)", vec);
+  if (a->batch > 1 && (a->stride_qb < a->n_q * a->stride_qn || a->stride_kb < a->n_k * a->stride_kn))
+    return fail(FHOG_E_STRIDE, "batch stride smaller than one (n, d) slice");
+  for (int i = 0; i < 14; i++)
+    if (!aligned16(ptrs[i])) return fail(FHOG_E_ALIGN, "pointer '%s' is not 16-byte aligned", names[i]);
+  if (a->impl == FHOG_IMPL_BF16) {
+    if (a->dtype != FHOG_DTYPE_BF16) return fail(FHOG_E_DTYPE, "impl=bf16 needs bf16 tensors");
+    if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
+      return fail(FHOG_E_SHAPE, "impl=bf16 needs d in {64,128} and n_q, n_k multiples of 128");
+  }
+  return FHOG_OK;
+}
+
+int select_impl(const fhog_bwdbwd_args* a) {
+  if (a->impl == FHOG_IMPL_FP32) return FHOG_IMPL_FP32;
+  if (a->impl == FHOG_IMPL_BF16) return FHOG_IMPL_BF16;
+  if (a->dtype == FHOG_DTYPE_BF16 && fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal)) return FHOG_IMPL_BF16;
+  return FHOG_IMPL_FP32;
+}
+
+fhog::Params to_params(const fhog_bwdbwd_args* a) {
+  fhog::Params p;
+  p.q = a->q;
+  p.k = a->k;
+  p.v = a->v;
+  p.o = a->o;
+  p.dO = a->dO;
+  p.ddq = a->ddq;
+  p.ddk = a->ddk;
+  p.ddv = a->ddv;
+  p.lse = a->lse;
+  p.dq2 = a->dq2;
+  p.dk2 = a->dk2;
+  p.dv2 = a->dv2;
+  p.ddo = a->ddo;
+  const int64_t rows = a->batch * a->n_q;
+  p.ws_d = a->ws;
+  p.ws_dd = a->ws + rows;
+  p.ws_b = a->ws + 2 * rows;
+  p.stride_qb = a->stride_qb;
+  p.stride_qn = a->stride_qn;
+  p.stride_kb = a->stride_kb;
+  p.stride_kn = a->stride_kn;
+  p.batch = (int32_t)a->batch;
+  p.n_q = (int32_t)a->n_q;
+  p.n_k = (int32_t)a->n_k;
+  p.d = (int32_t)a->d;
+  p.scale = a->scale;
+  p.causal = a->causal;
+  return p;
+}
+
+int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& p, int impl, int pass, hipStream_t s) {
+  hipError_t e;
+  if (pass == FHOG_PASS_D)
+    e = fhog::launch_rowdot(p, a->dtype, s);
+  else if (impl == FHOG_IMPL_BF16)
+    e = fhog::launch_bf16_pass(p, pass, s);
+  else
+    e = fhog::launch_fp32_pass(p, a->dtype, pass, s);
+  if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "pass %d: HIP error %d (%s)", pass, (int)e, hipGetErrorString(e));
+  return FHOG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fhog_abi_version(void) { return FHOG_ABI_VERSION; }
+
+size_t fhog_bwdbwd_args_size(void) { return sizeof(fhog_bwdbwd_args); }
+
+size_t fhog_bwdbwd_workspace_bytes(int64_t batch, int64_t n_q) {
+  if (batch < 0 || n_q < 0) return 0;
+  return (size_t)3 * (size_t)batch * (size_t)n_q * sizeof(float);
+}
+
+int fhog_validate(const fhog_bwdbwd_args* args) { return validate(args); }
+
+int fhog_select_impl(const fhog_bwdbwd_args* args) {
+  const int rc = validate(args);
+  if (rc != FHOG_OK) return rc;
+  return select_impl(args);
+}
+
+int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream) {
+  const int rc = validate(args);
+  if (rc != FHOG_OK) return rc;
+  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DK_DV) return fail(FHOG_E_PASS, "unknown pass %d", pass);
+  const fhog::Params p = to_params(args);
+  return run_pass(args, p, select_impl(args), pass, (hipStream_t)hip_stream);
+}
+
+int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
+  const int rc = validate(args);
+  if (rc != FHOG_OK) return rc;
+  const fhog::Params p = to_params(args);
+  const int impl = select_impl(args);
+  for (int pass = FHOG_PASS_D; pass <= FHOG_PASS_DK_DV; pass++) {
+    const int r = run_pass(args, p, impl, pass, (hipStream_t)hip_stream);
+    if (r != FHOG_OK) return r;
+  }
+  return FHOG_OK;
+}
+
+const char* fhog_last_error(void) { return g_err; }
+
+}  // extern "C"

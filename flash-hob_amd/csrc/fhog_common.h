@@ -1,0 +1,50 @@
+// Shared device/host declarations of libfhog_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fhog_hip.h"
+
+namespace fhog {
+
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Kernel-side view of fhog_bwdbwd_args (same fields, typed for device code).
+struct Params {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* o;
+  const void* dO;
+  const void* ddq;
+  const void* ddk;
+  const void* ddv;
+  const float* lse;
+  void* dq2;
+  void* dk2;
+  void* dv2;
+  void* ddo;
+  float* ws_d;   // (batch, n_q)
+  float* ws_dd;  // (batch, n_q)
+  float* ws_b;   // (batch, n_q)
+  int64_t stride_qb, stride_qn, stride_kb, stride_kn;
+  int32_t batch, n_q, n_k, d;
+  float scale;
+  int32_t causal;
+};
+
+// Launchers implemented in the kernel translation units. Each returns hipGetLastError().
+hipError_t launch_rowdot(const Params& p, int dtype, hipStream_t s);                 // pass 0
+hipError_t launch_fp32_pass(const Params& p, int dtype, int pass, hipStream_t s);   // passes 1..4, fp32 MFMA
+hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s);              // passes 1..4, bf16 MFMA
+bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal);
+
+}  // namespace fhog

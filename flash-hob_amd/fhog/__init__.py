@@ -1,0 +1,8 @@
+"""MI355X-native Flash Hog: attention double-backward on hand-written gfx950 kernels.
+
+Public entry point mirrors the reference package (``fhog/__init__.py:1-3``).
+"""
+from .bwdbwd import BwdBwdPlan, flash_bwdbwd
+from .attention import AttnBwd, FlashAttention, attention, attention_forward, produce_L
+
+__all__ = ["flash_bwdbwd", "BwdBwdPlan", "FlashAttention", "AttnBwd", "attention", "attention_forward", "produce_L"]

@@ -1,0 +1,150 @@
+"""Autograd surface around the double-backward kernels.
+
+The reference sketches this chain but never finishes it: ``FlashAttention2`` saves
+``(q, k, v, output, L)`` and ``is_causal`` (``fhog/triton_flash.py:136-198``) and the
+``Bwd`` Function that would route ``create_graph=True`` into ``flash_bwdbwd`` is a
+commented stub (``fhog/triton_bwdbwd.py:538-554``).  Here it is wired:
+
+    FlashAttention.forward   -> O, saves (q, k, v, O, L)
+    FlashAttention.backward  -> AttnBwd.apply(q, k, v, O, dO, L, scale, causal)
+    AttnBwd.forward          -> dQ, dK, dV   (first-order backward)
+    AttnBwd.backward         -> flash_bwdbwd(...) -> dQ', dK', dV', ddO
+
+The forward and the first-order backward are the callers on either side of the hot path;
+they are linear-memory torch compositions (blocked over heads and query rows, fp32
+accumulation), not tuned kernels.  The double-backward is the HIP library.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .bwdbwd import flash_bwdbwd
+
+_BLOCK_ELEMS = 1 << 26  # fp32 elements of one materialised (heads, rows, N_K) block (256 MiB)
+
+
+def _blocks(batch: int, n_q: int, n_k: int):
+    """Yield (head slice, row slice) so that heads*rows*n_k stays below the block budget."""
+    rows = max(1, min(n_q, _BLOCK_ELEMS // max(1, n_k)))
+    heads = max(1, min(batch, _BLOCK_ELEMS // (rows * n_k)))
+    for b0 in range(0, batch, heads):
+        for r0 in range(0, n_q, rows):
+            yield slice(b0, min(batch, b0 + heads)), slice(r0, min(n_q, r0 + rows))
+
+
+def _scores(q, k, scale, causal, r0):
+    s = torch.matmul(q.float(), k.float().transpose(-1, -2)) * scale
+    if causal:
+        n_r, n_k = s.shape[-2], s.shape[-1]
+        qi = torch.arange(r0, r0 + n_r, device=s.device)[:, None]
+        kj = torch.arange(n_k, device=s.device)[None, :]
+        s = s.masked_fill(kj > qi, float("-inf"))
+    return s
+
+
+def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = False):
+    """O (dtype of q) and fp32 L = logsumexp_j(scale q.k_j) for (batch, N, d) tensors.
+
+    Takes the place of the reference's forward kernel outputs (``fhog/triton_flash.py:123-133``)
+    and of ``produce_L`` (``fhog/triton_flash.py:252-258``), with causal support and without an
+    (batch, N_Q, N_K) allocation.
+    """
+    if q.dim() == 4:
+        B, H = q.shape[:2]
+        o, L = attention_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), scale, causal)
+        return o.view(q.shape), L.view(B, H, -1)
+    batch, n_q, d = q.shape
+    n_k = k.shape[1]
+    if causal and n_q != n_k:
+        raise ValueError("causal needs N_Q == N_K")
+    scale = d ** -0.5 if scale is None else scale
+    o = torch.empty_like(q)
+    L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
+    for hs, rs in _blocks(batch, n_q, n_k):
+        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start)
+        lse = torch.logsumexp(s, dim=-1)
+        p = torch.exp(s - lse[..., None])
+        o[hs, rs] = torch.matmul(p, v[hs].float()).to(q.dtype)
+        L[hs, rs] = lse
+    return o, L
+
+
+def produce_L(Q, K, is_causal: bool = False):
+    """fp32 log-sum-exp of ``Q K^T / sqrt(d)``; same call as ``fhog/triton_flash.py:252-258``
+    (which raises on causal and returns the input dtype)."""
+    return attention_forward(Q, K, K, None, is_causal)[1]
+
+
+def attention_backward(q, k, v, o, do, L, scale: float, causal: bool):
+    """First-order backward (dQ, dK, dV), blocked; the arithmetic of ``fhog/triton_flash.py:201-220``."""
+    batch, n_q, d = q.shape
+    n_k = k.shape[1]
+    dq = torch.empty_like(q)
+    dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
+    dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
+    for hs, rs in _blocks(batch, n_q, n_k):
+        qf, dof = q[hs, rs].float(), do[hs, rs].float()
+        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start)
+        p = torch.exp(s - L[hs, rs].float()[..., None])
+        dsum = (o[hs, rs].float() * dof).sum(-1, keepdim=True)
+        dp = torch.matmul(dof, v[hs].float().transpose(-1, -2))
+        ds = p * (dp - dsum) * scale
+        dq[hs, rs] = torch.matmul(ds, k[hs].float()).to(q.dtype)
+        dk[hs] += torch.matmul(ds.transpose(-1, -2), qf)
+        dv[hs] += torch.matmul(p.transpose(-1, -2), dof)
+    return dq, dk.to(k.dtype), dv.to(v.dtype)
+
+
+class AttnBwd(torch.autograd.Function):
+    """First-order attention backward as a differentiable node; its backward is the HIP double-backward.
+
+    Signature follows the reference's stub ``Bwd.forward(ctx, Q, K, V, dO, L, scale)``
+    (``fhog/triton_bwdbwd.py:538-554``) plus the cached ``O`` and the causal flag.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k, v, o, do, L, scale, causal):
+        ctx.save_for_backward(q, k, v, o, do, L)
+        ctx.scale = scale
+        ctx.causal = causal
+        sq = q.shape
+        f = (lambda t: t.flatten(0, 1)) if q.dim() == 4 else (lambda t: t)
+        dq, dk, dv = attention_backward(f(q), f(k), f(v), f(o), f(do), f(L), scale, causal)
+        return dq.view(sq), dk.view(k.shape), dv.view(v.shape)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, ddq, ddk, ddv):
+        q, k, v, o, do, L = ctx.saved_tensors
+        dq2, dk2, dv2, ddo = flash_bwdbwd(q, k, v, o, do, ddq.contiguous(), ddk.contiguous(), ddv.contiguous(), L,
+                                          ctx.scale, causal=ctx.causal)
+        # O and L are caches of (q, k, v): the four results are already total derivatives.
+        return dq2, dk2, dv2, None, ddo, None, None, None
+
+
+class FlashAttention(torch.autograd.Function):
+    """``FlashAttention.apply(q, k, v, is_causal)`` - call-compatible with the reference's
+    ``FlashAttention2`` (``fhog/triton_flash.py:136-198``), twice differentiable."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, is_causal=False):
+        scale = q.shape[-1] ** -0.5
+        o, L = attention_forward(q, k, v, scale, is_causal)
+        ctx.save_for_backward(q, k, v, o, L)
+        ctx.is_causal = is_causal
+        ctx.scale = scale
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, L = ctx.saved_tensors
+        dq, dk, dv = AttnBwd.apply(q, k, v, o, do.contiguous(), L, ctx.scale, ctx.is_causal)
+        return dq, dk, dv, None
+
+
+def attention(q, k, v, is_causal: bool = False):
+    """Twice-differentiable scaled-dot-product attention (scale = d^-1/2)."""
+    return FlashAttention.apply(q, k, v, is_causal)

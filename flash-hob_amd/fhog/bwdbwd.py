@@ -1,0 +1,184 @@
+"""Host wrapper of the attention double-backward: same entry point as the reference's
+``flash_bwdbwd`` (``fhog/triton_bwdbwd.py:557-648``), backed by ``libfhog_hip.so``.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32}
+_IMPLS = {None: _lib.IMPL_AUTO, "auto": _lib.IMPL_AUTO, "fp32": _lib.IMPL_FP32, "bf16": _lib.IMPL_BF16}
+
+
+def _flatten(t: torch.Tensor, name: str) -> torch.Tensor:
+    """(batch, N, d) stays; (B, H, N, d) becomes (B*H, N, d) (a view when possible)."""
+    if t.dim() == 3:
+        return t
+    if t.dim() == 4:
+        return t.reshape(t.shape[0] * t.shape[1], t.shape[2], t.shape[3])
+    raise ValueError(f"{name}: expected a 3-D (batch, N, d) or 4-D (B, H, N, d) tensor, got shape {tuple(t.shape)}")
+
+
+def _same_layout(ts) -> bool:
+    s0 = ts[0].stride()
+    return all(t.stride() == s0 for t in ts)
+
+
+def _prepare_group(ts, names):
+    """Tensors of one group must share (batch stride, row stride) and have a contiguous last dim."""
+    vec = 16 // ts[0].element_size()
+    ok = (_same_layout(ts) and ts[0].stride(2) == 1 and ts[0].stride(1) >= ts[0].shape[2]
+          and ts[0].stride(1) % vec == 0 and ts[0].stride(0) % vec == 0
+          and (ts[0].shape[0] == 1 or ts[0].stride(0) >= ts[0].shape[1] * ts[0].stride(1))
+          and all(t.data_ptr() % 16 == 0 for t in ts))
+    if ok:
+        return list(ts)
+    return [t.contiguous() for t in ts]
+
+
+def workspace_floats(batch: int, n_q: int) -> int:
+    return _lib.lib().fhog_bwdbwd_workspace_bytes(batch, n_q) // 4
+
+
+def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws) -> _lib.BwdBwdArgs:
+    a = _lib.BwdBwdArgs()
+    a.q, a.k, a.v, a.o, a.dO = Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dO.data_ptr()
+    a.ddq, a.ddk, a.ddv = ddQ.data_ptr(), ddK.data_ptr(), ddV.data_ptr()
+    a.lse = L.data_ptr()
+    a.dq2, a.dk2, a.dv2, a.ddo = (t.data_ptr() for t in outs)
+    a.ws = ws.data_ptr()
+    a.batch, a.n_q, a.d = Q.shape
+    a.n_k = K.shape[1]
+    a.stride_qb, a.stride_qn = Q.stride(0), Q.stride(1)
+    a.stride_kb, a.stride_kn = K.stride(0), K.stride(1)
+    a.scale = float(scale)
+    a.dtype = _DTYPES[Q.dtype]
+    a.causal = int(bool(causal))
+    a.impl = impl
+    return a
+
+
+def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = False, impl: Optional[str] = None,
+                 return_stats: bool = False, only_pass: Optional[int] = None):
+    """Flash Higher-Order-Gradients: VJP of the attention backward pass.
+
+    Same positional signature and return order as the reference
+    (``fhog/triton_bwdbwd.py:558,648``)::
+
+        dQ2, dK2, dV2, ddO = flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale)
+
+    Args:
+        Q, O, dO, ddQ: (batch, N_Q, d) or (B, H, N_Q, d); K, V, ddK, ddV: (batch, N_K, d) or (B, H, N_K, d).
+            bf16 or fp32 (all the same dtype), on a ROCm device.
+        L: (batch, N_Q) / (B, H, N_Q) log-sum-exp of ``scale * Q K^T`` over visible keys. Used in fp32
+            (any other dtype is up-cast; the reference passes it in the input dtype,
+            ``fhog/triton_flash.py:255-257``).
+        scale: python float.
+        causal: keyword only; top-left mask, needs N_Q == N_K. (The reference has no causal
+            double-backward.)
+        impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the bf16 MFMA kernels for
+            bf16 tensors whose shape they support, the fp32-MFMA kernels otherwise.
+        return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
+        only_pass: run a single pass (0..4) instead of all five; for tests and profiling.
+
+    Returns:
+        dQ2, dK2, dV2, ddO shaped and typed like Q, K, V, O (+ ``(d, dd, b)`` if ``return_stats``).
+    """
+    tensors = dict(Q=Q, K=K, V=V, O=O, dO=dO, ddQ=ddQ, ddK=ddK, ddV=ddV)
+    for n, t in tensors.items():
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{n} must be a torch.Tensor, got {type(t).__name__}")
+    if not isinstance(L, torch.Tensor):
+        raise TypeError(f"L must be a torch.Tensor, got {type(L).__name__}")
+    if Q.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {Q.dtype}; expected torch.bfloat16 or torch.float32")
+    for n, t in tensors.items():
+        if t.dtype != Q.dtype:
+            raise TypeError(f"{n} has dtype {t.dtype}, expected {Q.dtype} like Q")
+        if t.device != Q.device:
+            raise ValueError(f"{n} is on {t.device}, expected {Q.device} like Q")
+    if impl not in _IMPLS:
+        raise ValueError(f"impl must be one of {sorted(k for k in _IMPLS if k)} or None, got {impl!r}")
+    out_shape_q, out_shape_k = Q.shape, K.shape
+    q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = (_flatten(t, n) for n, t in tensors.items())
+    batch, n_q, d = q3.shape
+    n_k = k3.shape[1]
+    for n, t in (("O", o3), ("dO", do3), ("ddQ", ddq3)):
+        if t.shape != q3.shape:
+            raise ValueError(f"{n} has shape {tuple(t.shape)}, expected {tuple(q3.shape)} like Q")
+    if k3.shape[0] != batch or k3.shape[2] != d:
+        raise ValueError(f"K has shape {tuple(k3.shape)}, expected ({batch}, N_K, {d})")
+    for n, t in (("V", v3), ("ddK", ddk3), ("ddV", ddv3)):
+        if t.shape != k3.shape:
+            raise ValueError(f"{n} has shape {tuple(t.shape)}, expected {tuple(k3.shape)} like K")
+    if L.numel() != batch * n_q:
+        raise ValueError(f"L has {L.numel()} elements, expected batch*N_Q = {batch * n_q}")
+    if d not in (32, 64, 128):
+        raise ValueError(f"head dim {d} not supported (32, 64 or 128)")
+    if causal and n_q != n_k:
+        raise ValueError(f"causal needs N_Q == N_K, got {n_q} and {n_k}")
+    if not Q.is_cuda:
+        raise ValueError("flash_bwdbwd runs on the GPU only: tensors must be on a ROCm device (there is no CPU path)")
+    lse = L.reshape(batch, n_q)
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        lse = lse.to(torch.float32).contiguous()
+
+    q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
+    k3, v3, ddk3, ddv3 = _prepare_group([k3, v3, ddk3, ddv3], "k")
+
+    with torch.cuda.device(Q.device):
+        dq2 = torch.empty_strided(q3.shape, q3.stride(), dtype=Q.dtype, device=Q.device)
+        ddo = torch.empty_strided(q3.shape, q3.stride(), dtype=Q.dtype, device=Q.device)
+        dk2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
+        dv2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
+        ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
+        args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl],
+                           (dq2, dk2, dv2, ddo), ws)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        L_ = _lib.lib()
+        if only_pass is None:
+            _lib.check(L_.fhog_bwdbwd(ctypes.byref(args), stream))
+        else:
+            _lib.check(L_.fhog_bwdbwd_pass(ctypes.byref(args), int(only_pass), stream))
+    res = (dq2.view(out_shape_q) if dq2.is_contiguous() else dq2.reshape(out_shape_q),
+           dk2.view(out_shape_k) if dk2.is_contiguous() else dk2.reshape(out_shape_k),
+           dv2.view(out_shape_k) if dv2.is_contiguous() else dv2.reshape(out_shape_k),
+           ddo.view(out_shape_q) if ddo.is_contiguous() else ddo.reshape(out_shape_q))
+    if return_stats:
+        st = ws.view(3, *L.shape)
+        return res + ((st[0], st[1], st[2]),)
+    return res
+
+
+class BwdBwdPlan:
+    """Pre-validated call with caller-owned outputs and workspace (no allocation per call).
+
+    For benchmark loops and per-pass profiling; ``flash_bwdbwd`` is the drop-in entry point.
+    """
+
+    def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, impl=None):
+        ts = [_flatten(t, "tensor") for t in (Q, K, V, O, dO, ddQ, ddK, ddV)]
+        q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = ts
+        q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
+        k3, v3, ddk3, ddv3 = _prepare_group([k3, v3, ddk3, ddv3], "k")
+        batch, n_q, _ = q3.shape
+        lse = L.reshape(batch, n_q).to(torch.float32).contiguous()
+        self.keep = (q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse)
+        self.outs = (torch.empty_like(q3), torch.empty_like(k3), torch.empty_like(v3), torch.empty_like(q3))
+        self.ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
+        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws)
+        self.lib = _lib.lib()
+        _lib.check(self.lib.fhog_validate(ctypes.byref(self.args)))
+        self.impl = self.lib.fhog_select_impl(ctypes.byref(self.args))
+
+    def run(self, stream: Optional[int] = None, only_pass: Optional[int] = None):
+        s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
+        if only_pass is None:
+            _lib.check(self.lib.fhog_bwdbwd(ctypes.byref(self.args), s))
+        else:
+            _lib.check(self.lib.fhog_bwdbwd_pass(ctypes.byref(self.args), int(only_pass), s))
+        return self.outs

@@ -1,0 +1,123 @@
+/*
+ * fhog_hip.h - C ABI of libfhog_hip.so, the MI355X (gfx950) attention double-backward.
+ *
+ * One call replaces the body of the reference's host wrapper
+ *   flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale) -> (dQ2, dK2, dV2, ddO)
+ *   (fhog/triton_bwdbwd.py:557-648): the row reduction D = sum(dO*O) (:580), the launch
+ *   of bwdbwd_kernel_stage1 (:586-612, kernels :33-313) and of bwdbwd_kernel_stage2
+ *   (:620-646, kernels :316-535).
+ *
+ * Rules of the boundary
+ *   - plain C: pointers, integers, floats; no C++ or torch types.
+ *   - the library never allocates or frees device memory; the caller owns inputs,
+ *     outputs and the workspace (fhog_bwdbwd_workspace_bytes).
+ *   - every function returns 0 on success or a negative FHOG_E_* code; nothing throws
+ *     or exits; fhog_last_error() gives a thread-local message for the last failure.
+ *   - kernels are enqueued on the caller's hipStream_t (passed as void*); the library
+ *     never synchronises.
+ *   - all tensors are row-major (batch, N, d) with the last dimension contiguous;
+ *     the row stride and batch stride (in elements) are given per tensor group.
+ */
+#ifndef FHOG_HIP_H
+#define FHOG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FHOG_ABI_VERSION 1
+
+/* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
+#define FHOG_DTYPE_BF16 0
+#define FHOG_DTYPE_FP32 1
+
+/* error codes */
+#define FHOG_OK 0
+#define FHOG_E_NULL (-1)      /* a required pointer is NULL */
+#define FHOG_E_SHAPE (-2)     /* batch/n_q/n_k/d not supported */
+#define FHOG_E_DTYPE (-3)     /* unknown dtype */
+#define FHOG_E_STRIDE (-4)    /* stride smaller than the row / not a multiple of the vector width */
+#define FHOG_E_ALIGN (-5)     /* pointer not 16-byte aligned */
+#define FHOG_E_CAUSAL (-6)    /* causal with n_q != n_k */
+#define FHOG_E_PASS (-7)      /* unknown pass id */
+#define FHOG_E_LAUNCH (-8)    /* HIP reported an error at launch */
+#define FHOG_E_SCALE (-9)     /* scale is not finite */
+
+/* pass ids for fhog_bwdbwd_pass */
+#define FHOG_PASS_D 0      /* d_i  = sum_c O_ic dO_ic                         (fhog/triton_bwdbwd.py:580)     */
+#define FHOG_PASS_DD 1     /* dd_i = sum_j ddS_ij P_ij                        (fhog/triton_bwdbwd.py:185-211) */
+#define FHOG_PASS_B 2      /* b_i  = sum_j dP'_ij P_ij                        (fhog/triton_bwdbwd.py:217-251) */
+#define FHOG_PASS_DQ_DDO 3 /* dQ2 = dS ddK + dS' K ; ddO = P ddV + ddP V      (fhog/triton_bwdbwd.py:257-313) */
+#define FHOG_PASS_DK_DV 4  /* dK2 = dS^T ddQ + dS'^T Q ; dV2 = ddP^T dO       (fhog/triton_bwdbwd.py:467-535) */
+
+/* kernel families (fhog_bwdbwd_args.impl) */
+#define FHOG_IMPL_AUTO 0   /* bf16 MFMA kernels when the shape allows, else the fp32-MFMA kernels */
+#define FHOG_IMPL_FP32 1   /* force the fp32-MFMA kernels (any dtype; every intermediate in fp32) */
+#define FHOG_IMPL_BF16 2   /* force the bf16 MFMA kernels; error if the shape/dtype does not fit */
+
+typedef struct fhog_bwdbwd_args {
+  /* inputs (device pointers); q, o, dO, ddq: (batch, n_q, d); k, v, ddk, ddv: (batch, n_k, d) */
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* o;
+  const void* dO;
+  const void* ddq;
+  const void* ddk;
+  const void* ddv;
+  const float* lse; /* (batch, n_q) fp32, contiguous: L_i = logsumexp_j(scale * q_i . k_j) over unmasked j */
+  /* outputs (device pointers), same dtype and strides as the matching input group */
+  void* dq2; /* like q */
+  void* dk2; /* like k */
+  void* dv2; /* like k */
+  void* ddo; /* like q */
+  /* workspace: 3 * batch * n_q floats, laid out d | dd | b, each (batch, n_q) contiguous */
+  float* ws;
+  int64_t batch, n_q, n_k, d;
+  /* element strides. The q group (q, o, dO, ddq, dq2, ddo) shares stride_qb/stride_qn,
+     the k group (k, v, ddk, ddv, dk2, dv2) shares stride_kb/stride_kn; last-dim stride is 1. */
+  int64_t stride_qb, stride_qn, stride_kb, stride_kn;
+  float scale;
+  int32_t dtype;  /* FHOG_DTYPE_* */
+  int32_t causal; /* 0 | 1 (top-left mask: key j visible to query i iff j <= i; needs n_q == n_k) */
+  int32_t impl;   /* FHOG_IMPL_* */
+  int32_t reserved;
+} fhog_bwdbwd_args;
+
+/* Version of this header the library was built from. */
+int fhog_abi_version(void);
+
+/* sizeof(fhog_bwdbwd_args) as the library sees it, so that a foreign-language binding can check its mirror. */
+size_t fhog_bwdbwd_args_size(void);
+
+/* Bytes of workspace fhog_bwdbwd needs: 3 * batch * n_q * sizeof(float).
+   Replaces the torch allocations of D, dD, B at fhog/triton_bwdbwd.py:580-584. */
+size_t fhog_bwdbwd_workspace_bytes(int64_t batch, int64_t n_q);
+
+/* Host-only argument check (no HIP call is made; works without a GPU).
+   Returns FHOG_OK or the FHOG_E_* code fhog_bwdbwd would return for these arguments. */
+int fhog_validate(const fhog_bwdbwd_args* args);
+
+/* Which kernel family fhog_bwdbwd would use for these arguments: FHOG_IMPL_FP32 or
+   FHOG_IMPL_BF16, or a negative FHOG_E_* code. Host-only. */
+int fhog_select_impl(const fhog_bwdbwd_args* args);
+
+/* All passes in order (d, dd, b, dQ2+ddO, dK2+dV2) on `hip_stream` (a hipStream_t).
+   Drop-in for the two launches + reduction of flash_bwdbwd (fhog/triton_bwdbwd.py:580-646). */
+int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
+
+/* One pass only (FHOG_PASS_*), for per-pass tests and profiling. Passes read the
+   workspace rows written by earlier passes (stage 2 of the reference reads dD, B, D the
+   same way: fhog/triton_bwdbwd.py:474-482). */
+int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream);
+
+/* Message for the last failing call on this thread ("" if none). */
+const char* fhog_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FHOG_HIP_H */

@@ -1,0 +1,147 @@
+"""CPU tier: the C-ABI library loads, exports every symbol the header declares, and rejects bad
+arguments on the host before any launch. No compute call is made here (no GPU needed)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def L():
+    from fhog import _lib
+    return _lib.lib()
+
+
+def good_args():
+    from fhog import _lib
+    a = _lib.BwdBwdArgs()
+    for i, (name, _) in enumerate(_lib.BwdBwdArgs._fields_[:14]):
+        setattr(a, name, 0x10000 * (i + 1))  # fake, 16-byte aligned device addresses (never dereferenced)
+    a.batch, a.n_q, a.n_k, a.d = 4, 256, 512, 64
+    a.stride_qn = a.stride_kn = 64
+    a.stride_qb, a.stride_kb = 256 * 64, 512 * 64
+    a.scale, a.dtype, a.causal, a.impl = 0.125, 0, 0, 0
+    return a
+
+
+def test_header_symbols_exported(L):
+    header = (ROOT / "include" / "fhog_hip.h").read_text()
+    names = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(fhog_\w+)\s*\(", header, flags=re.M)
+    assert set(names) >= {"fhog_abi_version", "fhog_bwdbwd_args_size", "fhog_bwdbwd_workspace_bytes", "fhog_validate", "fhog_select_impl",
+                          "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error"}
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_struct_mirror_matches_header():
+    from fhog import _lib
+    header = (ROOT / "include" / "fhog_hip.h").read_text()
+    body = header[header.index("typedef struct fhog_bwdbwd_args"):header.index("} fhog_bwdbwd_args;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for decl in body.split("{", 1)[1].split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for piece in decl.split(","):
+            fields.append(re.findall(r"(\w+)\s*$", piece.strip())[0])
+    assert fields == [f[0] for f in _lib.BwdBwdArgs._fields_]
+    assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 200
+
+
+def test_version_and_workspace(L):
+    assert L.fhog_abi_version() == 1
+    assert L.fhog_bwdbwd_workspace_bytes(32, 4096) == 3 * 32 * 4096 * 4
+    assert L.fhog_bwdbwd_workspace_bytes(-1, 5) == 0
+
+
+def test_validate_accepts_good(L):
+    a = good_args()
+    assert L.fhog_validate(ctypes.byref(a)) == 0
+    assert L.fhog_select_impl(ctypes.byref(a)) in (1, 2)
+    a.dtype = 1
+    a.stride_qn = a.stride_kn = 64
+    assert L.fhog_select_impl(ctypes.byref(a)) == 1  # fp32 tensors always take the fp32-MFMA family
+
+
+@pytest.mark.parametrize("mutate, code, word", [
+    (lambda a: setattr(a, "q", 0), -1, "q"),
+    (lambda a: setattr(a, "ws", 0), -1, "ws"),
+    (lambda a: setattr(a, "d", 96), -2, "head dim"),
+    (lambda a: setattr(a, "n_k", 0), -2, "n_k"),
+    (lambda a: setattr(a, "batch", 70000), -2, "batch"),
+    (lambda a: setattr(a, "dtype", 7), -3, "dtype"),
+    (lambda a: setattr(a, "impl", 9), -3, "impl"),
+    (lambda a: setattr(a, "stride_qn", 32), -4, "stride"),
+    (lambda a: setattr(a, "stride_kn", 68), -4, "multiples"),
+    (lambda a: setattr(a, "stride_qb", 64), -4, "batch stride"),
+    (lambda a: setattr(a, "k", 0x20004), -5, "aligned"),
+    (lambda a: setattr(a, "causal", 1), -6, "causal"),
+    (lambda a: setattr(a, "causal", 2), -6, "causal"),
+    (lambda a: setattr(a, "scale", float("nan")), -9, "scale"),
+])
+def test_validate_rejects(L, mutate, code, word):
+    a = good_args()
+    mutate(a)
+    assert L.fhog_validate(ctypes.byref(a)) == code
+    assert word in L.fhog_last_error().decode()
+    # the compute entry points refuse the same way, before any launch
+    assert L.fhog_bwdbwd(ctypes.byref(a), None) == code
+    assert L.fhog_bwdbwd_pass(ctypes.byref(a), 1, None) == code
+
+
+def test_null_args(L):
+    assert L.fhog_validate(None) == -1
+
+
+def test_impl_bf16_needs_bf16_shape(L):
+    a = good_args()
+    a.impl = 2
+    a.dtype = 1
+    assert L.fhog_validate(ctypes.byref(a)) == -3
+    a.dtype = 0
+    a.n_q = 100
+    a.stride_qb = 100 * 64
+    assert L.fhog_validate(ctypes.byref(a)) == -2
+
+
+def test_python_wrapper_errors():
+    import fhog
+    t = lambda *s, dt=torch.bfloat16: torch.zeros(*s, dtype=dt)
+    q, k = t(2, 64, 64), t(2, 128, 64)
+    L = torch.zeros(2, 64)
+    with pytest.raises(TypeError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k.float(), L, 0.125)
+    with pytest.raises(TypeError):
+        fhog.flash_bwdbwd(q.half(), k.half(), k.half(), q.half(), q.half(), q.half(), k.half(), k.half(), L, 0.125)
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, t(2, 64, 64), L, 0.125)
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125, causal=True)
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, torch.zeros(2, 63), 0.125)
+    with pytest.raises(ValueError, match="GPU only"):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125)  # CPU tensors: no CPU path exists
+    with pytest.raises(ValueError):
+        fhog.produce_L(q, t(2, 128, 64), is_causal=True)
+
+
+def test_product_does_not_import_oracle():
+    """The shipped package must not reach into oracle/ (it is the checker, not the product)."""
+    for f in (ROOT / "flash-hob_amd").rglob("*.py"):
+        assert "oracle" not in f.read_text(), f
+    for f in (ROOT / "flash-hob_amd" / "csrc").glob("*"):
+        assert "oracle" not in f.read_text(), f
+
+
+def test_workload_flop_counts():
+    from fhog.workloads import WORKLOADS
+    w = WORKLOADS["cfg2_bf16_causal_4096_d128"]
+    assert w.pairs == 32 * 4096 * 4097 // 2
+    assert abs(w.flops_algorithmic - 8.248e11) / 8.248e11 < 1e-3
+    assert abs(WORKLOADS["cfg1_bf16_nc_2048_d64"].flops_algorithmic - 4.123e11) / 4.123e11 < 1e-3
+    assert w.bytes_algorithmic == (256 * 2**20 + 32 * 4096 * 4) + 128 * 2**20
