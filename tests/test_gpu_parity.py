@@ -115,3 +115,152 @@ def test_strided_and_4d_inputs():
     for a, b in zip(outs, base):
         assert a.shape == (B, H, n, d)
         torch.testing.assert_close(a.reshape(B * H, n, d), b, rtol=0, atol=0)
+
+
+# ---------------------------------------------------------------- bf16 MFMA family
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 128, 128, 64), (3, 256, 256, 128), (2, 128, 384, 64), (9, 384, 128, 128),
+                                   (1, 512, 512, 128)])
+def test_bf16_family_small(shape, causal):
+    """bf16 MFMA kernels against the fp64 closed form, including the row vectors of passes 0..2."""
+    batch, n_q, n_k, d = shape
+    if causal:
+        n_k = n_q
+    x = make_case(batch, n_q, n_k, d, torch.bfloat16, seed=5, grad_std=0.1)
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal)
+    outs = run_fhog(x, scale, causal, impl="bf16", return_stats=True)
+    ref = reference_fp64_cpu(x, scale, causal)
+    e = errors(outs[:4], [ref[n] for n in NAMES])
+    assert max(e.values()) < 2e-2, e
+    for got, name in zip(outs[4], ("d", "dd", "b")):
+        assert normalised_max_error(got, ref[name]) < 1e-2, name
+    # the two kernel families agree far inside the gate
+    outs32 = run_fhog(x, scale, causal, impl="fp32")
+    e2 = errors(outs[:4], outs32)
+    assert max(e2.values()) < 1.5e-2, e2
+
+
+def test_bf16_auto_dispatch():
+    from fhog import BwdBwdPlan
+    x = with_caches(make_case(2, 256, 256, 64, torch.bfloat16, seed=6), 0.125, False)
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125)
+    assert plan.impl == 2
+    y = with_caches(make_case(2, 200, 256, 64, torch.bfloat16, seed=6), 0.125, False)
+    plan = BwdBwdPlan(y["Q"], y["K"], y["V"], y["O"], y["dO"], y["ddQ"], y["ddK"], y["ddV"], y["L"], 0.125)
+    assert plan.impl == 1
+
+
+def _full_config(name, seed, heads=None):
+    from fhog.workloads import WORKLOADS, make_inputs
+    w = WORKLOADS[name]
+    x = make_inputs(w, seed, device="cuda:0")
+    x = {n: t.flatten(0, 1) for n, t in x.items()}
+    x = with_caches(x, w.scale, w.causal)
+    outs = run_fhog(x, w.scale, w.causal)
+    hs = list(range(w.batch)) if heads is None else heads
+    worst = {}
+    for h0 in range(0, len(hs), 4):
+        sel = hs[h0:h0 + 4]
+        ref = reference_fp32_gpu(x, w.scale, w.causal, heads=sel)
+        e = errors([o[sel] for o in outs], ref)
+        worst = {n: max(worst.get(n, 0.0), v) for n, v in e.items()}
+    for o in outs:
+        assert torch.isfinite(o.float()).all()
+    return w, worst
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_cfg1_bf16_noncausal_2048_d64(seed):
+    w, e = _full_config("cfg1_bf16_nc_2048_d64", seed)
+    assert max(e.values()) < 2e-2, e
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_cfg2_bf16_causal_4096_d128_headline(seed):
+    w, e = _full_config("cfg2_bf16_causal_4096_d128", seed)
+    assert max(e.values()) < 2e-2, e
+
+
+def test_cfg3_bf16_causal_16384_d128_sampled_heads():
+    """configs[3]: all 32 heads run through the HIP path; 4 sampled heads are compared with the fp32 reference."""
+    w, e = _full_config("cfg3_bf16_causal_16384_d128", 0, heads=[0, 9, 18, 27])
+    assert max(e.values()) < 2e-2, e
+
+
+def test_cfg4_bf16_cross_attention_scaled_keys():
+    w, e = _full_config("cfg4_bf16_cross_1024x8192_d64", 0)
+    assert max(e.values()) < 2e-2, e
+
+
+# ---------------------------------------------------------------- size-independent properties at full size
+def test_headline_properties_linearity_zero_and_sdpa_case():
+    from fhog.workloads import WORKLOADS, make_inputs
+    w = WORKLOADS["cfg2_bf16_causal_4096_d128"]
+    x = {n: t.flatten(0, 1)[:8] for n, t in make_inputs(w, 2, device="cuda:0").items()}
+    x = with_caches(x, w.scale, True)
+    # zero cotangents -> exact zeros
+    z = dict(x, ddQ=torch.zeros_like(x["ddQ"]), ddK=torch.zeros_like(x["ddK"]), ddV=torch.zeros_like(x["ddV"]))
+    for o in run_fhog(z, w.scale, True):
+        assert o.float().abs().max().item() == 0.0
+    # linearity in the cotangents: f(2 t) == 2 f(t) exactly (powers of two commute with every rounding)
+    base = run_fhog(x, w.scale, True)
+    dbl = run_fhog(dict(x, ddQ=x["ddQ"] * 2, ddK=x["ddK"] * 2, ddV=x["ddV"] * 2), w.scale, True)
+    for a, b in zip(base, dbl):
+        torch.testing.assert_close(b.float(), a.float() * 2, rtol=0, atol=0)
+    # ddQ = ddK = 0: dV' = 0, ddO = attention(Q, K, ddV), (dQ', dK') = first-order grads with V := ddV
+    y = dict(x, ddQ=torch.zeros_like(x["ddQ"]), ddK=torch.zeros_like(x["ddK"]))
+    dq2, dk2, dv2, ddo = run_fhog(y, w.scale, True)
+    assert dv2.float().abs().max().item() == 0.0
+    q = x["Q"].float().requires_grad_(True)
+    k = x["K"].float().requires_grad_(True)
+    out = torch.nn.functional.scaled_dot_product_attention(q, k, x["ddV"].float(), is_causal=True, scale=w.scale)
+    gq, gk = torch.autograd.grad(out, (q, k), x["dO"].float())
+    assert normalised_max_error(ddo, out) < 2e-2
+    assert normalised_max_error(dq2, gq) < 2e-2
+    assert normalised_max_error(dk2, gk) < 2e-2
+    # causal row 0 sees only key 0: dQ'[0] = 0, ddO[0] = ddV[0]
+    assert base[0][:, 0].float().abs().max().item() < 1e-6
+    torch.testing.assert_close(base[3][:, 0].float(), x["ddV"][:, 0].float(), rtol=1e-2, atol=1e-3)
+
+
+def test_peak_memory_is_linear_in_n():
+    """Workspace + outputs only: 4 output tensors and 3 fp32 row vectors, nothing of size N_Q x N_K."""
+    import fhog
+    sizes = {}
+    for n in (2048, 8192):
+        x = with_caches(make_case(4, n, n, 128, torch.bfloat16, seed=7, grad_std=0.1), 128 ** -0.5, True)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        outs = run_fhog(x, 128 ** -0.5, True)
+        torch.cuda.synchronize()
+        sizes[n] = torch.cuda.max_memory_allocated() - before
+        expect = 4 * 4 * n * 128 * 2 + 3 * 4 * n * 4
+        assert sizes[n] <= expect * 1.05 + (1 << 20), (n, sizes[n], expect)
+        del outs, x
+    assert sizes[8192] <= 4.2 * sizes[2048]
+
+
+# ---------------------------------------------------------------- autograd chain
+@pytest.mark.parametrize("causal", [False, True])
+def test_autograd_chain_reaches_hip_double_backward(causal):
+    """create_graph=True through FlashAttention -> AttnBwd -> flash_bwdbwd (the wiring the reference only
+    sketches, fhog/triton_bwdbwd.py:538-554) against plain torch attention."""
+    import fhog
+    g = torch.Generator().manual_seed(8)
+    mk = lambda *s: torch.randn(*s, generator=g).cuda()
+    q, k, v = mk(2, 128, 64), mk(2, 128, 64), mk(2, 128, 64)
+    w = mk(2, 128, 64)
+
+    def penalty(attn):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = attn(qq, kk, vv)
+        gq, gk, gv = torch.autograd.grad((out * w).sum(), (qq, kk, vv), create_graph=True)
+        loss = gq.square().sum() + (gk * gv).sum()
+        return torch.autograd.grad(loss, (qq, kk, vv))
+
+    ours = penalty(lambda a, b, c: fhog.attention(a, b, c, causal))
+    ref = penalty(lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(a, b, c, is_causal=causal))
+    for a, b in zip(ours, ref):
+        assert normalised_max_error(a, b) < 1e-4
