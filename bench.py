@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Headline benchmark: attention double-backward on one MI355X.
+
+One "step" = one call of ``fhog.flash_bwdbwd`` (five launches: d, dd, b, dQ'+ddO, dK'+dV') on
+seeded synthetic tensors that are already resident in HBM.  The workload is the configuration the
+metric is quoted on: bf16 causal B=2 H=16 N=4096 d=128.
+
+Prints ONE JSON line.  ``value`` is the whole-path algorithmic throughput
+(24*d*pairs FLOP per step: the 12 contractions of the materialised formula, recomputation
+not counted).  ``roofline`` describes the dominant kernel (pass 3, dQ'+ddO) against the dense
+bf16 MFMA peak; ``cpu_baseline`` is the torch autograd double-backward timed on this box's
+host cores on a few heads of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT / "flash-hob_amd", ROOT):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA: 256 CU x 4096 FLOP/clk x 2.4 GHz
+PASS_NAMES = {0: "rowdot_kernel", 1: "q_sweep_bf16<pass 1: dd>", 2: "q_sweep_bf16<pass 2: b>",
+              3: "q_sweep_bf16<pass 3: dQ2, ddO>", 4: "k_sweep_bf16<pass 4: dK2, dV2>"}
+# contractions each kernel needs to produce its outputs from its inputs (2*d*pairs FLOP each)
+PASS_CONTRACTIONS = {0: 0, 1: 3, 2: 5, 3: 9, 4: 8}
+
+
+def event_time_ms(fn, iters):
+    import torch
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def cpu_baseline(w, x_cpu, heads, repeats):
+    """torch autograd double-backward (fp32, materialised, one head at a time) on the host cores."""
+    import torch
+    from oracle.bwdbwd_oracle import autograd_double_backward
+    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
+    sel = {n: t[:heads].float() for n, t in x_cpu.items()}
+    args = (sel["Q"], sel["K"], sel["V"], sel["dO"], sel["ddQ"], sel["ddK"], sel["ddV"], w.scale, w.causal)
+    autograd_double_backward(*(a[:1] if torch.is_tensor(a) else a for a in args), dtype=torch.float32)  # warm-up, 1 head
+    best = float("inf")
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        autograd_double_backward(*args, dtype=torch.float32)
+        best = min(best, time.perf_counter() - t0)
+    flops = w.flops_algorithmic * heads / w.batch
+    return {"value": round(flops / best / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{heads} of {w.batch} (batch*head) slices of {w.name}, fp32 torch autograd double-backward on "
+                      f"materialised attention, best of {repeats}, {best:.2f} s",
+            "seconds": round(best, 3)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=None, help="one of fhog.workloads.WORKLOADS (default: the headline)")
+    ap.add_argument("--cpu-heads", type=int, default=32, help="slices of the workload timed on the CPU (0 = skip)")
+    ap.add_argument("--profile-only", action="store_true", help="run the timed loop only (for rocprofv3)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures ONE GPU (the path shards over batch*head with no communication); "
+                 "run with --gpus 1")
+
+    import torch
+    import fhog
+    from fhog.workloads import HEADLINE, WORKLOADS, make_inputs
+    from fhog import _lib
+    assert torch.cuda.is_available(), "bench.py needs a ROCm GPU"
+    _lib.lib()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    w = WORKLOADS[args.workload or HEADLINE]
+
+    x_cpu = {n: t.flatten(0, 1) for n, t in make_inputs(w, seed=0).items()}
+    x = {n: t.to(dev) for n, t in x_cpu.items()}
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)   # caches; not timed
+    call = lambda: fhog.flash_bwdbwd(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale,
+                                     causal=w.causal)
+    plan = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale, causal=w.causal)
+
+    for _ in range(args.warmup):
+        call()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base_mem = torch.cuda.memory_allocated()
+    ms = event_time_ms(call, args.steps)
+    peak_extra = torch.cuda.max_memory_allocated() - base_mem
+    peak_total = torch.cuda.max_memory_allocated()
+    if args.profile_only:
+        # a plain streaming kernel of known size (reads 256 MiB, writes 256 MiB) to calibrate byte counters
+        src = torch.zeros(64 * 2 ** 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        return
+
+    ms_plan = event_time_ms(plan.run, args.steps)
+    per_pass = {i: event_time_ms(lambda i=i: plan.run(only_pass=i), args.steps) for i in range(5)}
+    dom = max(per_pass, key=per_pass.get)
+    dom_flops = 2 * w.d * w.pairs * PASS_CONTRACTIONS[dom]
+    dom_tflops = dom_flops / per_pass[dom] / 1e9
+
+    value = w.flops_algorithmic / ms / 1e9
+    out = {
+        "metric": "double-bwd TFLOP/s, % bf16 MFMA peak @B2 H16 N4096 d128 causal; peak mem GB",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": w.name, "B": w.B, "H": w.H, "n_q": w.n_q, "n_k": w.n_k, "d": w.d, "causal": w.causal,
+                   "seed": 0, "kernel_family": {1: "fp32-mfma", 2: "bf16-mfma"}[plan.impl]},
+        "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+        "executed_tflops": round(w.flops_executed / ms / 1e9, 2),
+        "peak_mem_gb": round(peak_total / 1e9, 4),
+        "peak_mem_call_gb": round(peak_extra / 1e9, 4),
+        "ms_per_step_no_alloc": round(ms_plan, 4),
+        "ms_per_pass": {PASS_NAMES[i]: round(t, 4) for i, t in per_pass.items()},
+        "roofline": {"bound": "mfma", "kernel": PASS_NAMES[dom], "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4),
+                     "flops_per_launch": dom_flops, "ms_per_launch": round(per_pass[dom], 4),
+                     "traffic": TRAFFIC_BYTES.get((w.name, dom))},
+    }
+    if args.cpu_heads > 0:
+        out["cpu_baseline"] = cpu_baseline(w, x_cpu, min(args.cpu_heads, w.batch), repeats=2)
+    print(json.dumps(out))
+
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), keyed by (workload, pass). None until measured for that kernel.
+TRAFFIC_BYTES = {}
+
+if __name__ == "__main__":
+    main()
