@@ -15,107 +15,13 @@
 //     so each lane owns ONE stationary row: its row statistics are scalars, and the
 //     accumulator registers of the S-shaped tiles are directly the K-slots of the
 //     second-level MFMA operand (no shuffle, no LDS round trip).
-#include "fhog_common.h"
+#include <stdlib.h>
+
+#include "fhog_bf16_util.h"
 
 namespace fhog {
+using namespace bf16k;
 namespace {
-
-constexpr int WG_ROWS = 128;  // stationary rows per workgroup (4 waves x 32)
-constexpr int TS = 32;        // streamed rows per LDS stage
-constexpr int NSTAGE = 2;
-
-typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
-
-// ---- LDS tile addressing ------------------------------------------------------------------
-// A tile holds TS rows of D bf16 (2*D bytes per row, no padding). The 16-byte chunk `ch` of row
-// `r` is stored at chunk position ch ^ swz(r).
-template <int D>
-__device__ __forceinline__ int swz(int r) {
-  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
-  return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
-}
-template <int D>
-__device__ __forceinline__ int tile_off(int r, int ch) {
-  return r * (2 * D) + ((ch ^ swz<D>(r)) << 4);
-}
-
-__device__ __forceinline__ bf16x8_t lds_read128(const char* smem, int off) {
-  return *reinterpret_cast<const bf16x8_t*>(smem + off);
-}
-
-// Transposed operand: 8 K-slots for lane (col = lane%32, h = lane/32) of the 32-column block `cb`:
-// rows {16t + 4h + 0..3} and {16t + 8 + 4h + 0..3} of the tile at column cb*32 + lane%32.
-template <int D>
-__device__ __forceinline__ bf16x8_t lds_read_tr(const char* tile, int t, int cb, int lane) {
-  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
-  const int col = cb * 32 + 16 * b + 4 * (i & 3);
-  const int r0 = 16 * t + 4 * h + (i >> 2);
-  const int r1 = r0 + 8;
-  const int o0 = tile_off<D>(r0, col >> 3) + ((col >> 2) & 1) * 8;
-  const int o1 = tile_off<D>(r1, col >> 3) + ((col >> 2) & 1) * 8;
-  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o0));
-  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o1));
-  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-__device__ __forceinline__ f32x16_t mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-
-// registers 8t..8t+7 of an S-shaped fp32 tile -> the 8 K-slots of second-level step t
-__device__ __forceinline__ bf16x8_t pack8(const f32x16_t& x, int t) {
-  bf16x8_t r;
-#pragma unroll
-  for (int e = 0; e < 8; e++) r[e] = (__bf16)x[8 * t + e];
-  return r;
-}
-
-// ---- global -> register -> LDS staging of one 32-row tile set --------------------------------
-template <int D, int NT>
-struct Stage {
-  static constexpr int CPR = D / 8;                 // 16-byte chunks per row
-  static constexpr int PER_THREAD = TS * CPR / 256;  // chunks per thread per tensor (2 or 1)
-  u32x4_t v[NT][PER_THREAD];
-
-  __device__ __forceinline__ void load(const __bf16* const* src, int64_t ld, int row0, int tid) {
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-      for (int u = 0; u < PER_THREAD; u++) {
-        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
-        v[t][u] = *reinterpret_cast<const u32x4_t*>(src[t] + (int64_t)(row0 + r) * ld + ch * 8);
-      }
-  }
-  __device__ __forceinline__ void store(char* stage_base, int tid) const {
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-      for (int u = 0; u < PER_THREAD; u++) {
-        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
-        *reinterpret_cast<u32x4_t*>(stage_base + t * (TS * 2 * D) + tile_off<D>(r, ch)) = v[t][u];
-      }
-  }
-};
-
-// B operands of the stationary rows: lane (n = lane%32, h) holds row n, elements 16kk + 8h .. +7.
-template <int D>
-__device__ __forceinline__ void load_resident(bf16x8_t* dst, const __bf16* base, int64_t ld, int row, int h) {
-  const __bf16* p = base + (int64_t)row * ld + 8 * h;
-#pragma unroll
-  for (int kk = 0; kk < D / 16; kk++) dst[kk] = *reinterpret_cast<const bf16x8_t*>(p + 16 * kk);
-}
-
-// XCD-aware decode of a 1-D grid: workgroup ids go round-robin over the 8 XCDs, so all tiles of
-// one (batch*head) slice are given ids with the same id % 8 and share that XCD's L2.
-// Returns false when the id falls beyond the last slice.
-__device__ __forceinline__ bool decode_block(int n_tiles, int batch, bool heavy_first, int& bh, int& tile) {
-  const int id = blockIdx.x;
-  const int xcd = id & 7, slot = id >> 3;
-  bh = xcd + 8 * (slot / n_tiles);
-  tile = slot % n_tiles;
-  if (heavy_first) tile = n_tiles - 1 - tile;
-  return bh < batch;
-}
 
 // S-shaped results of one (32 streamed rows) x (32 stationary rows) block, as second-level operands.
 struct Ops {
@@ -467,8 +373,12 @@ bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
   return (d == 64 || d == 128) && n_q % WG_ROWS == 0 && n_k % WG_ROWS == 0;
 }
 
+hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s);
+
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
+  static const bool old_variant = getenv("FHOG_OLD34") != nullptr;
+  if (!old_variant && (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV)) return launch_bf16_pc_pass(p, pass, s);
   if (p.d == 128) return p.causal ? launch_d<128, true>(p, pass, s) : launch_d<128, false>(p, pass, s);
   return p.causal ? launch_d<64, true>(p, pass, s) : launch_d<64, false>(p, pass, s);
 }

@@ -1,0 +1,458 @@
+// Passes 3 (dQ2, ddO) and 4 (dK2, dV2) of the bf16 MFMA family as producer/consumer kernels.
+//
+// A workgroup is 512 threads = 8 wave64, two per SIMD, owning 128 stationary rows:
+//   producers (4 waves, 32 stationary rows each): first-level products of one 32x32 block
+//     (S, dP, ddS, dO ddV^T on MFMA), the softmax / dP' / dS / dS' / ddP arithmetic on the VALU,
+//     and the hand-off of the bf16 S-shaped operands through LDS;
+//   consumers (4 waves, same rows): the second-level products of the PREVIOUS block on MFMA
+//     (4 contractions in pass 3, 3 in pass 4) into the fp32 output accumulators, plus all
+//     global -> LDS staging of the streamed tiles.
+// The consumer runs one block behind the producer, so the VALU phase of the producer and the MFMA
+// phase of the consumer on the same SIMD overlap in hardware; each wave fits 256 registers.
+// One barrier per 32-row step. LDS: 3-stage ring of streamed tiles + double-buffered operand tiles.
+#include "fhog_bf16_util.h"
+
+namespace fhog {
+using namespace bf16k;
+namespace {
+
+constexpr int PC_THREADS = 512;
+constexpr int RING = 3;
+
+template <int D, bool PASS4>
+struct PCSmem {
+  static constexpr int NT = PASS4 ? 3 : 4;      // streamed tensors per stage
+  static constexpr int NSOP = PASS4 ? 3 : 4;    // operand tensors handed over per block
+  static constexpr int TILE = TS * 2 * D;
+  static constexpr int STAT = PASS4 ? 4 * TS * (int)sizeof(float) : 0;
+  static constexpr int STAGE = NT * TILE + STAT;
+  static constexpr int SOP_WAVE = NSOP * SOP_TILE;
+  static constexpr int SOP_BUF = 4 * SOP_WAVE;
+  static constexpr int SOP_BASE = RING * STAGE;
+  static constexpr int TOTAL = SOP_BASE + 2 * SOP_BUF;
+};
+
+// ---- pass 3 ------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
+                                          const bf16x8_t* dOb, int lane, int q_idx, int k_base, bool mask,
+                                          float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
+  constexpr int TILE = TS * 2 * D;
+  const int n = lane & 31, h = lane >> 5;
+  const char* tK = stage;
+  const char* tddK = stage + TILE;
+  const char* tV = stage + 2 * TILE;
+  const char* tddV = stage + 3 * TILE;
+  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
+  // LDS operands are fetched one k-step ahead of the MFMAs that use them
+  bf16x8_t a[2][4];
+  {
+    const int off = tile_off<D>(n, h);
+    a[0][0] = lds_read128(tK, off);
+    a[0][1] = lds_read128(tddK, off);
+    a[0][2] = lds_read128(tV, off);
+    a[0][3] = lds_read128(tddV, off);
+  }
+#pragma unroll
+  for (int kk = 0; kk < D / 16; kk++) {
+    const int c = kk & 1;
+    if (kk + 1 < D / 16) {
+      const int off = tile_off<D>(n, 2 * (kk + 1) + h);
+      a[c ^ 1][0] = lds_read128(tK, off);
+      a[c ^ 1][1] = lds_read128(tddK, off);
+      a[c ^ 1][2] = lds_read128(tV, off);
+      a[c ^ 1][3] = lds_read128(tddV, off);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    s = mfma(a[c][0], Qb[kk], s);
+    dds = mfma(a[c][0], ddQb[kk], dds);
+    dp = mfma(a[c][2], dOb[kk], dp);
+    dds = mfma(a[c][1], Qb[kk], dds);
+    e = mfma(a[c][3], dOb[kk], e);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  f32x16_t pv, dsv, ds2v, ddpv;
+#pragma unroll
+  for (int r = 0; r < 16; r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+  if (mask) {  // wave-uniform: only the block on the diagonal
+    const int lim = q_idx - k_base - 4 * h;
+#pragma unroll
+    for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const float p = pv[r];
+    const float ddsv = dds[r] * scale;
+    const float t1 = ddsv - dd;
+    const float dp2 = __builtin_fmaf(-ddsv, dsum, __builtin_fmaf(dp[r], t1, e[r]));
+    ddpv[r] = p * t1;
+    dsv[r] = p * (dp[r] - dsum);
+    ds2v[r] = p * (dp2 - b);
+  }
+  sop_write(sop + 0 * SOP_TILE, dsv, lane);
+  sop_write(sop + 1 * SOP_TILE, ds2v, lane);
+  sop_write(sop + 2 * SOP_TILE, ddpv, lane);
+  sop_write(sop + 3 * SOP_TILE, pv, lane);
+}
+
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  using SM = PCSmem<D, false>;
+  constexpr int NC = D / 32;
+
+  int bh, tile;
+  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bool producer = wave < 4;
+  const int wq = wave & 3;
+  const int n = lane & 31, h = lane >> 5;
+  const int q0 = tile * WG_ROWS, qw = q0 + 32 * wq, qi = qw + n;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
+
+  if (producer) {
+    bf16x8_t Qb[D / 16], ddQb[D / 16], dOb[D / 16];
+    load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
+    load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qi, h);
+    load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
+    const int64_t row = (int64_t)bh * p.n_q + qi;
+    const float l_log2 = p.lse[row] * kLog2e;
+    const float c_scale_log2 = p.scale * kLog2e;
+    const float dsum = p.ws_d[row], dd = p.ws_dd[row], b = p.ws_b[row];
+    __syncthreads();
+    int sp = 0;  // ring slot of tile j
+    for (int j = 0; j <= n_tiles; j++) {
+      const int k0 = j * TS;
+      if (j < n_tiles && (!CAUSAL || k0 <= qw)) {
+        const char* stage = smem + sp * SM::STAGE;
+        char* sop = sop_base + (j & 1) * SM::SOP_BUF;
+        produce_q<D>(stage, sop, Qb, ddQb, dOb, lane, qi, k0, CAUSAL && k0 == qw, c_scale_log2, l_log2, p.scale, dsum, dd, b);
+      }
+      __syncthreads();
+      sp = (sp == RING - 1) ? 0 : sp + 1;
+    }
+  } else {
+    const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
+                            (const __bf16*)p.ddv + koff};
+    f32x16_t acc_dq[NC], acc_ddo[NC];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      acc_dq[cb] = f32x16_t{0};
+      acc_ddo[cb] = f32x16_t{0};
+    }
+    int troff[NC][2];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      troff[cb][0] = tr_lane_off<D>(cb, 0, lane);
+      troff[cb][1] = tr_lane_off<D>(cb, 1, lane);
+    }
+    Dma<D> dma;
+    dma.init(p.stride_kn, wq, lane);
+    const uint32_t ring_lds = lds_addr(smem);
+#pragma unroll
+    for (int x = 0; x < 4; x++) dma.issue(ring_lds + x * SM::TILE, src[x], wq);
+    dma_wait();
+    __syncthreads();
+    int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
+    for (int j = 0; j <= n_tiles; j++) {
+      if (j + 1 < n_tiles) {
+        const uint32_t dst = ring_lds + sn * SM::STAGE;
+        const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
+#pragma unroll
+        for (int x = 0; x < 4; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
+      }
+      if (j >= 1 && (!CAUSAL || (j - 1) * TS <= qw)) {
+        const char* stage = smem + sc * SM::STAGE;
+        const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
+        const char* bp[NC][2];
+#pragma unroll
+        for (int cb = 0; cb < NC; cb++) {
+          bp[cb][0] = stage + troff[cb][0];
+          bp[cb][1] = stage + troff[cb][1];
+        }
+        bf16x8_t a_op[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int x = 0; x < 4; x++) a_op[t][x] = sop_read(sop + x * SOP_TILE, t, lane);
+        // B operands are fetched one (t, cb) step ahead of the MFMAs that use them
+        bf16x8_t bop[2][4];
+        bop[0][0] = lds_read_tr_pre(bp[0][0], bp[0][1], 1 * SM::TILE + 0 * 16 * 2 * D);
+        bop[0][1] = lds_read_tr_pre(bp[0][0], bp[0][1], 0 * SM::TILE + 0 * 16 * 2 * D);
+        bop[0][2] = lds_read_tr_pre(bp[0][0], bp[0][1], 2 * SM::TILE + 0 * 16 * 2 * D);
+        bop[0][3] = lds_read_tr_pre(bp[0][0], bp[0][1], 3 * SM::TILE + 0 * 16 * 2 * D);
+#pragma unroll
+        for (int it = 0; it < 2 * NC; it++) {
+          const int t = it / NC, cb = it % NC, c = it & 1;
+          if (it + 1 < 2 * NC) {
+            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+            bop[c ^ 1][0] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 1 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][1] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 0 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][2] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][3] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 3 * SM::TILE + t1 * 16 * 2 * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          acc_dq[cb] = mfma(a_op[t][0], bop[c][0], acc_dq[cb]);
+          acc_ddo[cb] = mfma(a_op[t][2], bop[c][2], acc_ddo[cb]);
+          acc_dq[cb] = mfma(a_op[t][1], bop[c][1], acc_dq[cb]);
+          acc_ddo[cb] = mfma(a_op[t][3], bop[c][3], acc_ddo[cb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      dma_wait();
+      __syncthreads();
+      sc = (sc == RING - 1) ? 0 : sc + 1;
+      sn = (sn == RING - 1) ? 0 : sn + 1;
+    }
+    // acc[cb][r] holds (query qw + 8*(r/4) + 4h + r%4, column cb*32 + n)
+    __bf16* odq = (__bf16*)p.dq2 + qoff;
+    __bf16* oddo = (__bf16*)p.ddo + qoff;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t o = (int64_t)(qw + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_qn + cb * 32 + n;
+        odq[o] = (__bf16)(acc_dq[cb][r] * p.scale);
+        oddo[o] = (__bf16)acc_ddo[cb][r];
+      }
+  }
+}
+
+// ---- pass 4 ------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* ddKb,
+                                          const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int k_idx, int q_base,
+                                          bool mask, float c_scale_log2, float scale) {
+  constexpr int TILE = TS * 2 * D;
+  const int n = lane & 31, h = lane >> 5;
+  const char* tQ = stage;
+  const char* tddQ = stage + TILE;
+  const char* tdO = stage + 2 * TILE;
+  const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
+  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
+  bf16x8_t a[2][3];
+  {
+    const int off = tile_off<D>(n, h);
+    a[0][0] = lds_read128(tQ, off);
+    a[0][1] = lds_read128(tddQ, off);
+    a[0][2] = lds_read128(tdO, off);
+  }
+#pragma unroll
+  for (int kk = 0; kk < D / 16; kk++) {
+    const int c = kk & 1;
+    if (kk + 1 < D / 16) {
+      const int off = tile_off<D>(n, 2 * (kk + 1) + h);
+      a[c ^ 1][0] = lds_read128(tQ, off);
+      a[c ^ 1][1] = lds_read128(tddQ, off);
+      a[c ^ 1][2] = lds_read128(tdO, off);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    s = mfma(a[c][0], Kb[kk], s);
+    dds = mfma(a[c][1], Kb[kk], dds);
+    dp = mfma(a[c][2], Vb[kk], dp);
+    dds = mfma(a[c][0], ddKb[kk], dds);
+    e = mfma(a[c][2], ddVb[kk], e);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  f32x16_t pv, dsv, ds2v, ddpv;
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 0 * TS + 8 * g + 4 * h);
+#pragma unroll
+    for (int j = 0; j < 4; j++) pv[4 * g + j] = __builtin_amdgcn_exp2f(s[4 * g + j] * c_scale_log2 - l4[j]);
+  }
+  if (mask) {  // wave-uniform: only the block on the diagonal
+    const int lim = k_idx - q_base - 4 * h;   // query row 8g + 4h + j sees key k_idx iff 8g + j >= lim
+#pragma unroll
+    for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) >= lim) ? pv[r] : 0.f;
+  }
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
+    const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
+    const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int r = 4 * g + j;
+      const float p = pv[r];
+      const float ddsv = dds[r] * scale;
+      const float t1 = ddsv - dd4[j];
+      const float dp2 = __builtin_fmaf(-ddsv, d4[j], __builtin_fmaf(dp[r], t1, e[r]));
+      ddpv[r] = p * t1;
+      dsv[r] = p * (dp[r] - d4[j]);
+      ds2v[r] = p * (dp2 - b4[j]);
+    }
+  }
+  sop_write(sop + 0 * SOP_TILE, dsv, lane);
+  sop_write(sop + 1 * SOP_TILE, ds2v, lane);
+  sop_write(sop + 2 * SOP_TILE, ddpv, lane);
+}
+
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  using SM = PCSmem<D, true>;
+  constexpr int NC = D / 32;
+
+  int bh, tile;
+  if (!decode_block(p.n_k / WG_ROWS, p.batch, false, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bool producer = wave < 4;
+  const int wq = wave & 3;
+  const int n = lane & 31, h = lane >> 5;
+  const int k0 = tile * WG_ROWS, kw = k0 + 32 * wq, kj = kw + n;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  // causal: query tiles before this workgroup's first key see none of its keys
+  const int t_begin = CAUSAL ? k0 / TS : 0;
+  const int t_end = p.n_q / TS;
+  char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
+
+  if (producer) {
+    bf16x8_t Kb[D / 16], ddKb[D / 16], Vb[D / 16], ddVb[D / 16];
+    load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kj, h);
+    load_resident<D>(ddKb, (const __bf16*)p.ddk + koff, p.stride_kn, kj, h);
+    load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kj, h);
+    load_resident<D>(ddVb, (const __bf16*)p.ddv + koff, p.stride_kn, kj, h);
+    const float c_scale_log2 = p.scale * kLog2e;
+    __syncthreads();
+    int sp = 0;  // ring slot of tile j (slot 0 holds tile t_begin)
+    for (int j = t_begin; j <= t_end; j++) {
+      const int qb = j * TS;
+      if (j < t_end && (!CAUSAL || qb >= kw)) {
+        const char* stage = smem + sp * SM::STAGE;
+        char* sop = sop_base + (j & 1) * SM::SOP_BUF;
+        produce_k<D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, kj, qb, CAUSAL && qb == kw, c_scale_log2, p.scale);
+      }
+      __syncthreads();
+      sp = (sp == RING - 1) ? 0 : sp + 1;
+    }
+  } else {
+    const int ctid = tid - 256;
+    const __bf16* src[3] = {(const __bf16*)p.q + qoff, (const __bf16*)p.ddq + qoff, (const __bf16*)p.dO + qoff};
+    const float* stat_src[4] = {p.lse + (int64_t)bh * p.n_q, p.ws_d + (int64_t)bh * p.n_q, p.ws_dd + (int64_t)bh * p.n_q,
+                                p.ws_b + (int64_t)bh * p.n_q};
+    f32x16_t acc_dk[NC], acc_dv[NC];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      acc_dk[cb] = f32x16_t{0};
+      acc_dv[cb] = f32x16_t{0};
+    }
+    int troff[NC][2];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      troff[cb][0] = tr_lane_off<D>(cb, 0, lane);
+      troff[cb][1] = tr_lane_off<D>(cb, 1, lane);
+    }
+    Dma<D> dma;
+    dma.init(p.stride_qn, wq, lane);
+    const uint32_t ring_lds = lds_addr(smem);
+    float stat_reg = 0.f;  // consumer threads 0..127: one statistic value of the staged tile
+    auto load_stat = [&](int q_base) {
+      if (ctid < 4 * TS) {
+        const float v = stat_src[ctid / TS][q_base + (ctid % TS)];
+        stat_reg = (ctid < TS) ? v * kLog2e : v;
+      }
+    };
+    auto store_stat = [&](char* stage_base) {
+      if (ctid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * SM::TILE)[ctid] = stat_reg;
+    };
+    {
+      const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
+#pragma unroll
+      for (int x = 0; x < 3; x++) dma.issue(ring_lds + x * SM::TILE, src[x] + adv, wq);
+      load_stat(t_begin * TS);
+      store_stat(smem);
+    }
+    dma_wait();
+    __syncthreads();
+    int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
+    for (int j = t_begin; j <= t_end; j++) {
+      if (j + 1 < t_end) {
+        const uint32_t dst = ring_lds + sn * SM::STAGE;
+        const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
+#pragma unroll
+        for (int x = 0; x < 3; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
+        load_stat((j + 1) * TS);
+      }
+      if (j > t_begin && (!CAUSAL || (j - 1) * TS >= kw)) {
+        const char* stage = smem + sc * SM::STAGE;
+        const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
+        const char* bp[NC][2];
+#pragma unroll
+        for (int cb = 0; cb < NC; cb++) {
+          bp[cb][0] = stage + troff[cb][0];
+          bp[cb][1] = stage + troff[cb][1];
+        }
+        bf16x8_t a_op[2][3];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int x = 0; x < 3; x++) a_op[t][x] = sop_read(sop + x * SOP_TILE, t, lane);
+        bf16x8_t bop[2][3];
+        bop[0][0] = lds_read_tr_pre(bp[0][0], bp[0][1], 1 * SM::TILE + 0 * 16 * 2 * D);
+        bop[0][1] = lds_read_tr_pre(bp[0][0], bp[0][1], 0 * SM::TILE + 0 * 16 * 2 * D);
+        bop[0][2] = lds_read_tr_pre(bp[0][0], bp[0][1], 2 * SM::TILE + 0 * 16 * 2 * D);
+#pragma unroll
+        for (int it = 0; it < 2 * NC; it++) {
+          const int t = it / NC, cb = it % NC, c = it & 1;
+          if (it + 1 < 2 * NC) {
+            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+            bop[c ^ 1][0] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 1 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][1] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 0 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][2] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          acc_dk[cb] = mfma(a_op[t][0], bop[c][0], acc_dk[cb]);
+          acc_dv[cb] = mfma(a_op[t][2], bop[c][2], acc_dv[cb]);
+          acc_dk[cb] = mfma(a_op[t][1], bop[c][1], acc_dk[cb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (j + 1 < t_end) store_stat(smem + sn * SM::STAGE);
+      dma_wait();
+      __syncthreads();
+      sc = (sc == RING - 1) ? 0 : sc + 1;
+      sn = (sn == RING - 1) ? 0 : sn + 1;
+    }
+    __bf16* odk = (__bf16*)p.dk2 + koff;
+    __bf16* odv = (__bf16*)p.dv2 + koff;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int64_t o = (int64_t)(kw + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_kn + cb * 32 + n;
+        odk[o] = (__bf16)(acc_dk[cb][r] * p.scale);
+        odv[o] = (__bf16)acc_dv[cb][r];
+      }
+  }
+}
+
+template <int D, bool CAUSAL>
+hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
+  const dim3 block(PC_THREADS);
+  const int heads8 = (p.batch + 7) / 8 * 8;
+  hipError_t e;
+  if (pass == FHOG_PASS_DQ_DDO) {
+    const int smem = PCSmem<D, false>::TOTAL;
+    e = hipFuncSetAttribute((const void*)q_sweep3_pc<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((q_sweep3_pc<D, CAUSAL>), dim3((unsigned)(heads8 * (p.n_q / WG_ROWS))), block, smem, s, p);
+  } else {
+    const int smem = PCSmem<D, true>::TOTAL;
+    e = hipFuncSetAttribute((const void*)k_sweep_pc<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((k_sweep_pc<D, CAUSAL>), dim3((unsigned)(heads8 * (p.n_k / WG_ROWS))), block, smem, s, p);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s) {
+  if (p.d == 128) return p.causal ? launch_pc_d<128, true>(p, pass, s) : launch_pc_d<128, false>(p, pass, s);
+  return p.causal ? launch_pc_d<64, true>(p, pass, s) : launch_pc_d<64, false>(p, pass, s);
+}
+
+}  // namespace fhog

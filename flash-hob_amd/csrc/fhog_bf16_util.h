@@ -1,0 +1,194 @@
+// Device helpers shared by the bf16 MFMA kernels (gfx950): LDS tile addressing with the 16-byte
+// XOR swizzle, row-wise and transposing LDS operand reads, global->LDS staging, XCD-aware grid decode.
+#pragma once
+#include "fhog_common.h"
+
+namespace fhog {
+namespace bf16k {
+
+constexpr int WG_ROWS = 128;  // stationary rows per workgroup (4 waves x 32)
+constexpr int TS = 32;        // streamed rows per LDS stage
+constexpr int NSTAGE = 2;
+
+typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
+
+// ---- LDS tile addressing ------------------------------------------------------------------
+// A tile holds TS rows of D bf16 (2*D bytes per row, no padding). The 16-byte chunk `ch` of row
+// `r` is stored at chunk position ch ^ swz(r).
+template <int D>
+__device__ __forceinline__ int swz(int r) {
+  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
+}
+template <int D>
+__device__ __forceinline__ int tile_off(int r, int ch) {
+  return r * (2 * D) + ((ch ^ swz<D>(r)) << 4);
+}
+
+__device__ __forceinline__ bf16x8_t lds_read128(const char* smem, int off) {
+  return *reinterpret_cast<const bf16x8_t*>(smem + off);
+}
+
+// Transposed operand: 8 K-slots for lane (col = lane%32, h = lane/32) of the 32-column block `cb`:
+// rows {16t + 4h + 0..3} and {16t + 8 + 4h + 0..3} of the tile at column cb*32 + lane%32.
+template <int D>
+__device__ __forceinline__ bf16x8_t lds_read_tr(const char* tile, int t, int cb, int lane) {
+  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
+  const int col = cb * 32 + 16 * b + 4 * (i & 3);
+  const int r0 = 16 * t + 4 * h + (i >> 2);
+  const int r1 = r0 + 8;
+  const int o0 = tile_off<D>(r0, col >> 3) + ((col >> 2) & 1) * 8;
+  const int o1 = tile_off<D>(r1, col >> 3) + ((col >> 2) & 1) * 8;
+  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o0));
+  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o1));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Same, with the K-slots in row order: rows 16t + 8h + 0..7 (operand partner of sop_read).
+template <int D>
+__device__ __forceinline__ bf16x8_t lds_read_tr_lin(const char* tile, int t, int cb, int lane) {
+  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
+  const int col = cb * 32 + 16 * b + 4 * (i & 3);
+  const int r0 = 16 * t + 8 * h + (i >> 2);
+  const int r1 = r0 + 4;
+  const int o0 = tile_off<D>(r0, col >> 3) + ((col >> 2) & 1) * 8;
+  const int o1 = tile_off<D>(r1, col >> 3) + ((col >> 2) & 1) * 8;
+  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o0));
+  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o1));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Same operand with the per-lane part of the address precomputed (it does not depend on t):
+//   tr_lane_off(cb, s) for s = 0 (rows 8h + 0..3) and s = 1 (rows 8h + 4..7); step t adds 16 rows.
+template <int D>
+__device__ __forceinline__ int tr_lane_off(int cb, int s, int lane) {
+  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
+  const int col = cb * 32 + 16 * b + 4 * (i & 3);
+  const int r = 8 * h + 4 * s + (i >> 2);
+  return tile_off<D>(r, col >> 3) + ((col >> 2) & 1) * 8;
+}
+// p0 / p1: stage base + tr_lane_off(cb, 0 / 1); `imm` = tensor offset + t * 16 rows (compile-time)
+__device__ __forceinline__ bf16x8_t lds_read_tr_pre(const char* p0, const char* p1, int imm) {
+  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p0 + imm));
+  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p1 + imm));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// ---- S-shaped bf16 operand tiles handed from producer to consumer waves through LDS ------------
+// 32 stationary rows x 32 streamed rows, 64 bytes per row, 16-byte chunks XOR-swizzled by (row>>2)&3.
+constexpr int SOP_TILE = 32 * 64;
+// producer: registers 4g..4g+3 of an S-shaped fp32 tile (streamed rows 8g + 4h + 0..3) of stationary row n
+__device__ __forceinline__ void sop_write(char* tile, const f32x16_t& x, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    bf16x4_t v;
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = (__bf16)x[4 * g + e];
+    *reinterpret_cast<bf16x4_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = v;
+  }
+}
+// consumer: A operand of second-level step t: stationary row n, streamed rows 16t + 8h + 0..7
+__device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+  return *reinterpret_cast<const bf16x8_t*>(tile + n * 64 + (((2 * t + h) ^ ((n >> 2) & 3)) << 4));
+}
+
+__device__ __forceinline__ f32x16_t mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// registers 8t..8t+7 of an S-shaped fp32 tile -> the 8 K-slots of second-level step t
+__device__ __forceinline__ bf16x8_t pack8(const f32x16_t& x, int t) {
+  bf16x8_t r;
+#pragma unroll
+  for (int e = 0; e < 8; e++) r[e] = (__bf16)x[8 * t + e];
+  return r;
+}
+
+// ---- global -> register -> LDS staging of one 32-row tile set --------------------------------
+template <int D, int NT>
+struct Stage {
+  static constexpr int CPR = D / 8;                 // 16-byte chunks per row
+  static constexpr int PER_THREAD = TS * CPR / 256;  // chunks per thread per tensor (2 or 1)
+  u32x4_t v[NT][PER_THREAD];
+
+  __device__ __forceinline__ void load(const __bf16* const* src, int64_t ld, int row0, int tid) {
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int u = 0; u < PER_THREAD; u++) {
+        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
+        v[t][u] = *reinterpret_cast<const u32x4_t*>(src[t] + (int64_t)(row0 + r) * ld + ch * 8);
+      }
+  }
+  __device__ __forceinline__ void store(char* stage_base, int tid) const {
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int u = 0; u < PER_THREAD; u++) {
+        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
+        *reinterpret_cast<u32x4_t*>(stage_base + t * (TS * 2 * D) + tile_off<D>(r, ch)) = v[t][u];
+      }
+  }
+};
+
+// ---- direct global -> LDS staging (no registers): global_load_lds_dwordx4 ------------------------
+// One wave instruction moves 64 x 16 bytes to 1 KiB of contiguous LDS at M0 (lane l lands at
+// M0 + 16*l). The destination is therefore linear; the swizzle is applied on the SOURCE side: the lane
+// that lands on chunk position pc of row r fetches chunk pc ^ swz(r) of that row.
+// The load is issued from inline asm, so the compiler does not track it: the caller must execute
+// dma_wait() before the barrier that publishes the tile.
+template <int D>
+struct Dma {
+  static constexpr int CPR = D / 8;             // 16-byte chunks per row
+  static constexpr int RPI = 64 / CPR;          // rows per instruction (4 at d=128, 8 at d=64)
+  static constexpr int IPT = TS / RPI;          // instructions per 32-row tile (8 or 4)
+  static constexpr int PER_WAVE = IPT / 4;      // instructions per tile for each of 4 loader waves (2 or 1)
+  uint32_t voff[PER_WAVE];                      // per-lane byte offset from the tile's first row
+
+  __device__ __forceinline__ void init(int64_t ld, int lw, int lane) {
+#pragma unroll
+    for (int u = 0; u < PER_WAVE; u++) {
+      const int q = lw + 4 * u;
+      const int r = q * RPI + lane / CPR, pc = lane % CPR;
+      voff[u] = (uint32_t)((r * ld + ((pc ^ swz<D>(r)) << 3)) * 2);
+    }
+  }
+  // tile_lds: LDS byte address of the destination tile (wave-uniform); src: first row of the source tile
+  __device__ __forceinline__ void issue(uint32_t tile_lds, const __bf16* src, int lw) const {
+#pragma unroll
+    for (int u = 0; u < PER_WAVE; u++) {
+      const uint32_t m0 = __builtin_amdgcn_readfirstlane(tile_lds + (lw + 4 * u) * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(voff[u]), "s"(src) : "memory", "m0");
+    }
+  }
+};
+__device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ uint32_t lds_addr(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// B operands of the stationary rows: lane (n = lane%32, h) holds row n, elements 16kk + 8h .. +7.
+template <int D>
+__device__ __forceinline__ void load_resident(bf16x8_t* dst, const __bf16* base, int64_t ld, int row, int h) {
+  const __bf16* p = base + (int64_t)row * ld + 8 * h;
+#pragma unroll
+  for (int kk = 0; kk < D / 16; kk++) dst[kk] = *reinterpret_cast<const bf16x8_t*>(p + 16 * kk);
+}
+
+// XCD-aware decode of a 1-D grid: workgroup ids go round-robin over the 8 XCDs, so all tiles of
+// one (batch*head) slice are given ids with the same id % 8 and share that XCD's L2.
+// Returns false when the id falls beyond the last slice.
+__device__ __forceinline__ bool decode_block(int n_tiles, int batch, bool heavy_first, int& bh, int& tile) {
+  const int id = blockIdx.x;
+  const int xcd = id & 7, slot = id >> 3;
+  bh = xcd + 8 * (slot / n_tiles);
+  tile = slot % n_tiles;
+  if (heavy_first) tile = n_tiles - 1 - tile;
+  return bh < batch;
+}
+
+
+}  // namespace bf16k
+}  // namespace fhog
