@@ -28,7 +28,8 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
 
   int bh, tile;
   if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
@@ -70,49 +71,74 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
     const int k0 = j * TS;
     if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
       const char* stage = smem + (j & 1) * STAGE;
-      f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
-      // LDS operands are fetched one k-step ahead of the MFMAs that use them
-      bf16x8_t a[2][NT];
+      // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
+      // is cut into small pieces placed right behind the MFMAs of the same wave, where it runs in the
+      // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
+      //   K  : S += K Q^T, ddS += K ddQ^T
+      //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
+      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale, t = dP dd   (pass 2)
+      //   ddV: E += ddV dO^T           + acc += P (ddS u - t)                      (pass 2)
+      //   tail: acc += P ddS (pass 1) | acc += P E (pass 2)
+      constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
+      constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
+      f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
+      bf16x8_t a[NB];
 #pragma unroll
-      for (int x = 0; x < NT; x++) a[0][x] = lds_read128(stage + x * TILE, aoff[0]);
+      for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + kTensorOfPhase[i / KK] * TILE, aoff[i % KK]);
 #pragma unroll
-      for (int kk = 0; kk < KK; kk++) {
-        const int c = kk & 1;
-        if (kk + 1 < KK) {
-#pragma unroll
-          for (int x = 0; x < NT; x++) a[c ^ 1][x] = lds_read128(stage + x * TILE, aoff[kk + 1]);
-        }
+      for (int i = 0; i < NSTEP; i++) {
+        const int ph = (PASS == 1 && i >= KK) ? 2 : i / KK, kk = i % KK, c = i % NB;
+        if (i + PF < NSTEP)
+          a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
         __builtin_amdgcn_sched_barrier(0);
-        s = mfma(a[c][0], Qb[kk], s);
-        dds = mfma(a[c][0], ddQb[kk], dds);
-        if (PASS == 2) dp = mfma(a[c][NT - 2], dOb[kk], dp);
-        dds = mfma(a[c][1], Qb[kk], dds);
-        if (PASS == 2) e = mfma(a[c][NT - 1], dOb[kk], e);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      f32x16_t pv;
+        if (ph == 0) {
+          s = mfma(a[c], Qb[kk], s);
+          dds = mfma(a[c], ddQb[kk], dds);
+        } else if (ph == 1) {
+          dp = mfma(a[c], dOb[kk], dp);
 #pragma unroll
-      for (int r = 0; r < 16; r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
-      if (CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
-        const int lim = qi - k0 - 4 * h;
+          for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+        } else if (ph == 2) {
+          dds = mfma(a[c], Qb[kk], dds);
 #pragma unroll
-        for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
-      }
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float ddsv = dds[r] * p.scale;
-        if (PASS == 1) {
-          red = __builtin_fmaf(pv[r], ddsv, red);
+          for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
+            if (PASS == 1) {
+              pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+            } else {
+              us[r] = (dp[r] - dsum) * p.scale;
+              tt[r] = dp[r] * dd;
+            }
+          }
         } else {
-          const float dp2 = __builtin_fmaf(-ddsv, dsum, __builtin_fmaf(dp[r], ddsv - dd, e[r]));
-          red = __builtin_fmaf(pv[r], dp2, red);
+          e = mfma(a[c], dOb[kk], e);
+          if (kk == 0 && CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
+            const int lim = qi - k0 - 4 * h;
+#pragma unroll
+            for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+          }
+#pragma unroll
+          for (int r = EPK * kk; r < EPK * (kk + 1); r++) red = __builtin_fmaf(pv[r], __builtin_fmaf(dds[r], us[r], -tt[r]), red);
         }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (PASS == 1) {
+        if (CAUSAL && k0 == qw) {
+          const int lim = qi - k0 - 4 * h;
+#pragma unroll
+          for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], dds[r], red);   // scale applied once at the end
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
       }
     }
     dma_wait();
     __syncthreads();
   }
   red += __shfl_xor(red, 32);
+  if (PASS == 1) red *= p.scale;
   if (h == 0) (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
 }
 

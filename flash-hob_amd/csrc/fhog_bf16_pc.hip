@@ -33,67 +33,102 @@ struct PCSmem {
 };
 
 // ---- pass 3 ------------------------------------------------------------------------------------------
+// One 32-key x 32-query block of pass 3 on a producer wave.
+// The five first-level products are issued as a stream of 32 k-steps (8 each for K, V, ddK, ddV);
+// the elementwise work of the block is cut into 2-element pieces that are placed right behind the
+// MFMAs in the SAME wave's instruction stream, where they execute in the shadow of the matrix pipe
+// (VALU work of another wave does not overlap an MFMA on this hardware; work of the same wave does):
+//   steps  0.. 7  A = K  : S += K Q^T, ddS += K ddQ^T
+//   steps  8..15  A = V  : dP += V dO^T          + P = exp2(S c - L)
+//   steps 16..23  A = ddK: ddS += ddK Q^T        + u = dP - d, dS = P u, v = dP dd + b
+//   steps 24..31  A = ddV: E += ddV dO^T         + ddP = P (ddS - dd), z = P (ddS u - v)
+//   tail                                          dS' = P E + z     [= P (E + dP (ddS - dd) - ddS d - b)]
+// LDS operands are fetched PF steps ahead. Results go to the operand tiles dS, dS', ddP, P.
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  bf16x2_t v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+// registers 4g..4g+3 of one S-shaped tile, given as packed pairs pk[2g], pk[2g+1]
+__device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    u32x2_t v = {pk[2 * g], pk[2 * g + 1]};
+    *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = v;
+  }
+}
+
 template <int D>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
                                           const bf16x8_t* dOb, int lane, int q_idx, int k_base, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
   constexpr int TILE = TS * 2 * D;
+  constexpr int KK = D / 16, NSTEP = 4 * KK, PF = 2, NB = PF + 1;
   const int n = lane & 31, h = lane >> 5;
-  const char* tK = stage;
-  const char* tddK = stage + TILE;
-  const char* tV = stage + 2 * TILE;
-  const char* tddV = stage + 3 * TILE;
-  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
-  // LDS operands are fetched one k-step ahead of the MFMAs that use them
-  bf16x8_t a[2][4];
-  {
-    const int off = tile_off<D>(n, h);
-    a[0][0] = lds_read128(tK, off);
-    a[0][1] = lds_read128(tddK, off);
-    a[0][2] = lds_read128(tV, off);
-    a[0][3] = lds_read128(tddV, off);
-  }
+  int aoff[KK];
 #pragma unroll
-  for (int kk = 0; kk < D / 16; kk++) {
-    const int c = kk & 1;
-    if (kk + 1 < D / 16) {
-      const int off = tile_off<D>(n, 2 * (kk + 1) + h);
-      a[c ^ 1][0] = lds_read128(tK, off);
-      a[c ^ 1][1] = lds_read128(tddK, off);
-      a[c ^ 1][2] = lds_read128(tV, off);
-      a[c ^ 1][3] = lds_read128(tddV, off);
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+  // stream order of the A operands: K, V, ddK, ddV (stage order is K, ddK, V, ddV)
+  constexpr int kTensorOfPhase[4] = {0, 2, 1, 3};
+  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
+  f32x16_t pv, vv, us;
+  uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];
+  bf16x8_t a[NB];
+#pragma unroll
+  for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + kTensorOfPhase[i / KK] * TILE, aoff[i % KK]);
+
+  constexpr int EPK = 16 / KK;  // elements of the 16-register tiles handled per k-step (2 at d=128, 4 at d=64)
+#pragma unroll
+  for (int i = 0; i < NSTEP; i++) {
+    const int ph = i / KK, kk = i % KK, c = i % NB;
+    if (i + PF < NSTEP) a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ph == 0) {
+      s = mfma(a[c], Qb[kk], s);
+      dds = mfma(a[c], ddQb[kk], dds);
+    } else if (ph == 1) {
+      dp = mfma(a[c], dOb[kk], dp);
+#pragma unroll
+      for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+    } else if (ph == 2) {
+      dds = mfma(a[c], Qb[kk], dds);
+      if (kk == 0 && mask) {  // wave-uniform: only the block on the diagonal
+        const int lim = q_idx - k_base - 4 * h;
+#pragma unroll
+        for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+      }
+#pragma unroll
+      for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
+        const float u0 = dp[r] - dsum, u1 = dp[r + 1] - dsum;
+        pk_ds[r / 2] = pack2(pv[r] * u0, pv[r + 1] * u1);
+        vv[r] = __builtin_fmaf(dp[r], dd, b);
+        vv[r + 1] = __builtin_fmaf(dp[r + 1], dd, b);
+        us[r] = u0 * scale;
+        us[r + 1] = u1 * scale;
+      }
+    } else {
+      e = mfma(a[c], dOb[kk], e);
+#pragma unroll
+      for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
+        pk_ddp[r / 2] = pack2(pv[r] * __builtin_fmaf(dds[r], scale, -dd), pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd));
+        pk_p[r / 2] = pack2(pv[r], pv[r + 1]);
+        vv[r] = pv[r] * __builtin_fmaf(dds[r], us[r], -vv[r]);              // z
+        vv[r + 1] = pv[r + 1] * __builtin_fmaf(dds[r + 1], us[r + 1], -vv[r + 1]);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
-    s = mfma(a[c][0], Qb[kk], s);
-    dds = mfma(a[c][0], ddQb[kk], dds);
-    dp = mfma(a[c][2], dOb[kk], dp);
-    dds = mfma(a[c][1], Qb[kk], dds);
-    e = mfma(a[c][3], dOb[kk], e);
-    __builtin_amdgcn_sched_barrier(0);
   }
-  f32x16_t pv, dsv, ds2v, ddpv;
+  sop_write_pk(sop + 0 * SOP_TILE, pk_ds, lane);
+  sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, lane);
+  sop_write_pk(sop + 3 * SOP_TILE, pk_p, lane);
 #pragma unroll
-  for (int r = 0; r < 16; r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
-  if (mask) {  // wave-uniform: only the block on the diagonal
-    const int lim = q_idx - k_base - 4 * h;
-#pragma unroll
-    for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
-  }
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const float p = pv[r];
-    const float ddsv = dds[r] * scale;
-    const float t1 = ddsv - dd;
-    const float dp2 = __builtin_fmaf(-ddsv, dsum, __builtin_fmaf(dp[r], t1, e[r]));
-    ddpv[r] = p * t1;
-    dsv[r] = p * (dp[r] - dsum);
-    ds2v[r] = p * (dp2 - b);
-  }
-  sop_write(sop + 0 * SOP_TILE, dsv, lane);
-  sop_write(sop + 1 * SOP_TILE, ds2v, lane);
-  sop_write(sop + 2 * SOP_TILE, ddpv, lane);
-  sop_write(sop + 3 * SOP_TILE, pv, lane);
+  for (int r = 0; r < 16; r += 2)
+    pk_ds2[r / 2] = pack2(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
+  sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, lane);
 }
+
 
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
@@ -103,7 +138,8 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 
   int bh, tile;
   if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
   const int wq = wave & 3;
   const int n = lane & 31, h = lane >> 5;
@@ -134,20 +170,28 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       sp = (sp == RING - 1) ? 0 : sp + 1;
     }
   } else {
+    // consumer wave cw owns the 64 x 64 output block (query pair qp, column half ch): every transposed
+    // K-side operand read from LDS feeds two MFMAs (one per 32-query block of the pair)
+    const int qp = wq >> 1, ch = wq & 1;
     const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
                             (const __bf16*)p.ddv + koff};
-    f32x16_t acc_dq[NC], acc_ddo[NC];
+    f32x16_t acc_dq[2][2], acc_ddo[2][2];  // [query block of the pair][32-column block of the half]
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++) {
-      acc_dq[cb] = f32x16_t{0};
-      acc_ddo[cb] = f32x16_t{0};
-    }
-    int troff[NC][2];
+    for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++) {
-      troff[cb][0] = tr_lane_off<D>(cb, 0, lane);
-      troff[cb][1] = tr_lane_off<D>(cb, 1, lane);
+      for (int cl = 0; cl < 2; cl++) {
+        acc_dq[qb][cl] = f32x16_t{0};
+        acc_ddo[qb][cl] = f32x16_t{0};
+      }
+    int troff[2][2];
+#pragma unroll
+    for (int cl = 0; cl < 2; cl++) {
+      troff[cl][0] = tr_lane_off<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 0, lane);
+      troff[cl][1] = tr_lane_off<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 1, lane);
     }
+    constexpr int NCL = (D == 128) ? 2 : 1;  // 32-column blocks per consumer wave
+    const int qw0 = q0 + 64 * qp;            // first query of the pair
+    const char* sop_pair = smem + SM::SOP_BASE + (2 * qp) * SM::SOP_WAVE;
     Dma<D> dma;
     dma.init(p.stride_kn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
@@ -163,42 +207,56 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 #pragma unroll
         for (int x = 0; x < 4; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
       }
-      if (j >= 1 && (!CAUSAL || (j - 1) * TS <= qw)) {
+      // block j-1: query block qb of the pair took part iff its first query is not before the tile
+      const bool act0 = j >= 1 && (!CAUSAL || (j - 1) * TS <= qw0);
+      const bool act1 = j >= 1 && (!CAUSAL || (j - 1) * TS <= qw0 + 32);
+      if (act1) {  // act0 implies act1
         const char* stage = smem + sc * SM::STAGE;
-        const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
-        const char* bp[NC][2];
+        const char* sop = sop_pair + ((j - 1) & 1) * SM::SOP_BUF;
+        const char* bp[NCL][2];
 #pragma unroll
-        for (int cb = 0; cb < NC; cb++) {
-          bp[cb][0] = stage + troff[cb][0];
-          bp[cb][1] = stage + troff[cb][1];
+        for (int cl = 0; cl < NCL; cl++) {
+          bp[cl][0] = stage + troff[cl][0];
+          bp[cl][1] = stage + troff[cl][1];
         }
-        bf16x8_t a_op[2][4];
+        // operand order in the stage: K, ddK, V, ddV; in the operand tiles: dS, dS', ddP, P
+        bf16x8_t bop[2][4];
+#pragma unroll
+        for (int x = 0; x < 4; x++) bop[0][x] = lds_read_tr_pre(bp[0][0], bp[0][1], x * SM::TILE);
+        bf16x8_t a_opt[2][2][4];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int x = 0; x < 4; x++) a_op[t][x] = sop_read(sop + x * SOP_TILE, t, lane);
-        // B operands are fetched one (t, cb) step ahead of the MFMAs that use them
-        bf16x8_t bop[2][4];
-        bop[0][0] = lds_read_tr_pre(bp[0][0], bp[0][1], 1 * SM::TILE + 0 * 16 * 2 * D);
-        bop[0][1] = lds_read_tr_pre(bp[0][0], bp[0][1], 0 * SM::TILE + 0 * 16 * 2 * D);
-        bop[0][2] = lds_read_tr_pre(bp[0][0], bp[0][1], 2 * SM::TILE + 0 * 16 * 2 * D);
-        bop[0][3] = lds_read_tr_pre(bp[0][0], bp[0][1], 3 * SM::TILE + 0 * 16 * 2 * D);
+          for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-        for (int it = 0; it < 2 * NC; it++) {
-          const int t = it / NC, cb = it % NC, c = it & 1;
-          if (it + 1 < 2 * NC) {
-            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
-            bop[c ^ 1][0] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 1 * SM::TILE + t1 * 16 * 2 * D);
-            bop[c ^ 1][1] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 0 * SM::TILE + t1 * 16 * 2 * D);
-            bop[c ^ 1][2] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
-            bop[c ^ 1][3] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 3 * SM::TILE + t1 * 16 * 2 * D);
+            for (int x = 0; x < 4; x++) a_opt[t][qb][x] = sop_read(sop + qb * SM::SOP_WAVE + x * SOP_TILE, t, lane);
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const auto& a_op = a_opt[t];
+#pragma unroll
+          for (int cl = 0; cl < NCL; cl++) {
+            const int it = t * NCL + cl, c = it & 1;
+            if (it + 1 < 2 * NCL) {
+              const int t1 = (it + 1) / NCL, cl1 = (it + 1) % NCL;
+#pragma unroll
+              for (int x = 0; x < 4; x++)
+                bop[c ^ 1][x] = lds_read_tr_pre(bp[cl1][0], bp[cl1][1], x * SM::TILE + t1 * 16 * 2 * D);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (act0) {
+              acc_dq[0][cl] = mfma(a_op[0][0], bop[c][1], acc_dq[0][cl]);
+              acc_ddo[0][cl] = mfma(a_op[0][2], bop[c][2], acc_ddo[0][cl]);
+            }
+            acc_dq[1][cl] = mfma(a_op[1][0], bop[c][1], acc_dq[1][cl]);
+            acc_ddo[1][cl] = mfma(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
+            if (act0) {
+              acc_dq[0][cl] = mfma(a_op[0][1], bop[c][0], acc_dq[0][cl]);
+              acc_ddo[0][cl] = mfma(a_op[0][3], bop[c][3], acc_ddo[0][cl]);
+            }
+            acc_dq[1][cl] = mfma(a_op[1][1], bop[c][0], acc_dq[1][cl]);
+            acc_ddo[1][cl] = mfma(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
+            __builtin_amdgcn_sched_barrier(0);
           }
-          __builtin_amdgcn_sched_barrier(0);
-          acc_dq[cb] = mfma(a_op[t][0], bop[c][0], acc_dq[cb]);
-          acc_ddo[cb] = mfma(a_op[t][2], bop[c][2], acc_ddo[cb]);
-          acc_dq[cb] = mfma(a_op[t][1], bop[c][1], acc_dq[cb]);
-          acc_ddo[cb] = mfma(a_op[t][3], bop[c][3], acc_ddo[cb]);
-          __builtin_amdgcn_sched_barrier(0);
         }
       }
       dma_wait();
@@ -206,17 +264,19 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       sc = (sc == RING - 1) ? 0 : sc + 1;
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
-    // acc[cb][r] holds (query qw + 8*(r/4) + 4h + r%4, column cb*32 + n)
+    // acc[qb][cl][r] holds (query qw0 + 32 qb + 8*(r/4) + 4h + r%4, column 32*(NCL*ch + cl) + n)
     __bf16* odq = (__bf16*)p.dq2 + qoff;
     __bf16* oddo = (__bf16*)p.ddo + qoff;
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++)
+    for (int qb = 0; qb < 2; qb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int64_t o = (int64_t)(qw + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_qn + cb * 32 + n;
-        odq[o] = (__bf16)(acc_dq[cb][r] * p.scale);
-        oddo[o] = (__bf16)acc_ddo[cb][r];
-      }
+      for (int cl = 0; cl < NCL; cl++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int64_t o = (int64_t)(qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_qn + 32 * (NCL * ch + cl) + n;
+          odq[o] = (__bf16)(acc_dq[qb][cl][r] * p.scale);
+          oddo[o] = (__bf16)acc_ddo[qb][cl][r];
+        }
   }
 }
 
@@ -298,7 +358,8 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
 
   int bh, tile;
   if (!decode_block(p.n_k / WG_ROWS, p.batch, false, bh, tile)) return;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
   const int wq = wave & 3;
   const int n = lane & 31, h = lane >> 5;
