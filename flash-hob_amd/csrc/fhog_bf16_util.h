@@ -8,7 +8,6 @@ namespace bf16k {
 
 constexpr int WG_ROWS = 128;  // stationary rows per workgroup (4 waves x 32)
 constexpr int TS = 32;        // streamed rows per LDS stage
-constexpr int NSTAGE = 2;
 
 typedef __attribute__((address_space(3))) bf16x4_t* lds_bf16x4_ptr;
 
@@ -29,36 +28,11 @@ __device__ __forceinline__ bf16x8_t lds_read128(const char* smem, int off) {
   return *reinterpret_cast<const bf16x8_t*>(smem + off);
 }
 
-// Transposed operand: 8 K-slots for lane (col = lane%32, h = lane/32) of the 32-column block `cb`:
-// rows {16t + 4h + 0..3} and {16t + 8 + 4h + 0..3} of the tile at column cb*32 + lane%32.
-template <int D>
-__device__ __forceinline__ bf16x8_t lds_read_tr(const char* tile, int t, int cb, int lane) {
-  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
-  const int col = cb * 32 + 16 * b + 4 * (i & 3);
-  const int r0 = 16 * t + 4 * h + (i >> 2);
-  const int r1 = r0 + 8;
-  const int o0 = tile_off<D>(r0, col >> 3) + ((col >> 2) & 1) * 8;
-  const int o1 = tile_off<D>(r1, col >> 3) + ((col >> 2) & 1) * 8;
-  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o0));
-  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o1));
-  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// Same, with the K-slots in row order: rows 16t + 8h + 0..7 (operand partner of sop_read).
-template <int D>
-__device__ __forceinline__ bf16x8_t lds_read_tr_lin(const char* tile, int t, int cb, int lane) {
-  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
-  const int col = cb * 32 + 16 * b + 4 * (i & 3);
-  const int r0 = 16 * t + 8 * h + (i >> 2);
-  const int r1 = r0 + 4;
-  const int o0 = tile_off<D>(r0, col >> 3) + ((col >> 2) & 1) * 8;
-  const int o1 = tile_off<D>(r1, col >> 3) + ((col >> 2) & 1) * 8;
-  bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o0));
-  bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(tile + o1));
-  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// Same operand with the per-lane part of the address precomputed (it does not depend on t):
+// Transposed (second-level) operand of the 32-column block `cb`, read with ds_read_b64_tr_b16: lane
+// (col = lane%32, h = lane/32) receives the 8 K-slots = tile rows 16t + 8h + 0..7 at column
+// cb*32 + col. Two 8-byte transposing reads, one per group of 4 rows; within a 16-lane group lane i
+// addresses row (i>>2), columns 4*(i&3)..+3, and receives column i of the 4 x 16 block.
+// The per-lane part of the address does not depend on t and is precomputed:
 //   tr_lane_off(cb, s) for s = 0 (rows 8h + 0..3) and s = 1 (rows 8h + 4..7); step t adds 16 rows.
 template <int D>
 __device__ __forceinline__ int tr_lane_off(int cb, int s, int lane) {
@@ -97,41 +71,6 @@ __device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) 
 __device__ __forceinline__ f32x16_t mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
-
-// registers 8t..8t+7 of an S-shaped fp32 tile -> the 8 K-slots of second-level step t
-__device__ __forceinline__ bf16x8_t pack8(const f32x16_t& x, int t) {
-  bf16x8_t r;
-#pragma unroll
-  for (int e = 0; e < 8; e++) r[e] = (__bf16)x[8 * t + e];
-  return r;
-}
-
-// ---- global -> register -> LDS staging of one 32-row tile set --------------------------------
-template <int D, int NT>
-struct Stage {
-  static constexpr int CPR = D / 8;                 // 16-byte chunks per row
-  static constexpr int PER_THREAD = TS * CPR / 256;  // chunks per thread per tensor (2 or 1)
-  u32x4_t v[NT][PER_THREAD];
-
-  __device__ __forceinline__ void load(const __bf16* const* src, int64_t ld, int row0, int tid) {
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-      for (int u = 0; u < PER_THREAD; u++) {
-        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
-        v[t][u] = *reinterpret_cast<const u32x4_t*>(src[t] + (int64_t)(row0 + r) * ld + ch * 8);
-      }
-  }
-  __device__ __forceinline__ void store(char* stage_base, int tid) const {
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-      for (int u = 0; u < PER_THREAD; u++) {
-        const int c = tid + 256 * u, r = c / CPR, ch = c % CPR;
-        *reinterpret_cast<u32x4_t*>(stage_base + t * (TS * 2 * D) + tile_off<D>(r, ch)) = v[t][u];
-      }
-  }
-};
 
 // ---- direct global -> LDS staging (no registers): global_load_lds_dwordx4 ------------------------
 // One wave instruction moves 64 x 16 bytes to 1 KiB of contiguous LDS at M0 (lane l lands at
