@@ -102,7 +102,10 @@ int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& p, int impl, int pas
     e = fhog::launch_rowdot(p, a->dtype, s);
   else if (impl == FHOG_IMPL_BF16)
     e = fhog::launch_bf16_pass(p, pass, s);
-  else
+  else if (pass == FHOG_PASS_DD_B) {
+    e = fhog::launch_fp32_pass(p, a->dtype, FHOG_PASS_DD, s);
+    if (e == hipSuccess) e = fhog::launch_fp32_pass(p, a->dtype, FHOG_PASS_B, s);
+  } else
     e = fhog::launch_fp32_pass(p, a->dtype, pass, s);
   if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "pass %d: HIP error %d (%s)", pass, (int)e, hipGetErrorString(e));
   return FHOG_OK;
@@ -132,7 +135,7 @@ int fhog_select_impl(const fhog_bwdbwd_args* args) {
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream) {
   const int rc = validate(args);
   if (rc != FHOG_OK) return rc;
-  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DK_DV) return fail(FHOG_E_PASS, "unknown pass %d", pass);
+  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DD_B) return fail(FHOG_E_PASS, "unknown pass %d", pass);
   const fhog::Params p = to_params(args);
   return run_pass(args, p, select_impl(args), pass, (hipStream_t)hip_stream);
 }
@@ -142,7 +145,8 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   if (rc != FHOG_OK) return rc;
   const fhog::Params p = to_params(args);
   const int impl = select_impl(args);
-  for (int pass = FHOG_PASS_D; pass <= FHOG_PASS_DK_DV; pass++) {
+  const int order[] = {FHOG_PASS_D, FHOG_PASS_DD_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
+  for (int pass : order) {
     const int r = run_pass(args, p, impl, pass, (hipStream_t)hip_stream);
     if (r != FHOG_OK) return r;
   }

@@ -6,7 +6,11 @@
 //   pass 3  dQ2, ddO    Q-tiled   (fhog/triton_bwdbwd.py:257-313)   fhog_bf16_pc.hip
 //   pass 4  dK2, dV2    K-tiled   (fhog/triton_bwdbwd.py:467-535)   fhog_bf16_pc.hip
 //
-// Passes 1 and 2 (row statistics only): a workgroup is 256 threads = 4 wave64 owning 128 queries,
+// Fused statistics sweep (PASS = 5, what fhog_bwdbwd launches): b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
+// needs dd_i only as a factor of a row sum, so dd and b come out of ONE sweep with the five products of pass 2
+// and three running sums per query; the three products of a separate pass 1 are saved.
+//
+// Passes 1, 2 and 5 (row statistics only): a workgroup is 256 threads = 4 wave64 owning 128 queries,
 // two workgroups per CU. Each wave keeps its 32 query rows in registers as MFMA B operands
 // (Q, ddQ and, in pass 2, dO); K-side tiles of 32 keys stream through a two-stage LDS ring filled by
 // direct global->LDS loads. Products are computed transposed (keys = M, queries = N), so every lane
@@ -39,14 +43,14 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   bf16x8_t Qb[KK], ddQb[KK], dOb[KK];
   load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
   load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qi, h);
-  if (PASS == 2) load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
+  if (PASS != 1) load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
 
   const int64_t row = (int64_t)bh * p.n_q + qi;
   const float l_log2 = p.lse[row] * kLog2e;
   const float c_scale_log2 = p.scale * kLog2e;
-  const float dsum = PASS == 2 ? p.ws_d[row] : 0.f;
+  const float dsum = PASS != 1 ? p.ws_d[row] : 0.f;
   const float dd = PASS == 2 ? p.ws_dd[row] : 0.f;
-  float red = 0.f;
+  float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
 
   int aoff[KK];
 #pragma unroll
@@ -76,9 +80,10 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
       // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
       //   K  : S += K Q^T, ddS += K ddQ^T
       //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
-      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale, t = dP dd   (pass 2)
+      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale, t = dP dd   (pass 2; fused: u only)
       //   ddV: E += ddV dO^T           + acc += P (ddS u - t)                      (pass 2)
-      //   tail: acc += P ddS (pass 1) | acc += P E (pass 2)
+      //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
+      //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
       constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
       constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
       f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
@@ -106,7 +111,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
               pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
             } else {
               us[r] = (dp[r] - dsum) * p.scale;
-              tt[r] = dp[r] * dd;
+              if (PASS == 2) tt[r] = dp[r] * dd;
             }
           }
         } else {
@@ -117,7 +122,15 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
             for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
           }
 #pragma unroll
-          for (int r = EPK * kk; r < EPK * (kk + 1); r++) red = __builtin_fmaf(pv[r], __builtin_fmaf(dds[r], us[r], -tt[r]), red);
+          for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
+            if (PASS == 2) {
+              red = __builtin_fmaf(pv[r], __builtin_fmaf(dds[r], us[r], -tt[r]), red);
+            } else {
+              red_dd = __builtin_fmaf(pv[r], dds[r], red_dd);
+              red_pdp = __builtin_fmaf(pv[r], dp[r], red_pdp);
+              us[r] *= dds[r];
+            }
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -129,9 +142,12 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], dds[r], red);   // scale applied once at the end
-      } else {
+      } else if (PASS == 2) {
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], us[r] + e[r], red);
       }
     }
     dma_wait();
@@ -139,7 +155,17 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   }
   red += __shfl_xor(red, 32);
   if (PASS == 1) red *= p.scale;
-  if (h == 0) (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
+  if (PASS == 5) {
+    red_dd += __shfl_xor(red_dd, 32);
+    red_pdp += __shfl_xor(red_pdp, 32);
+    const float dd_i = red_dd * p.scale;
+    if (h == 0) {
+      p.ws_dd[row] = dd_i;
+      p.ws_b[row] = __builtin_fmaf(-dd_i, red_pdp, red);
+    }
+  } else if (h == 0) {
+    (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
+  }
 }
 
 template <int D, bool CAUSAL>
@@ -154,11 +180,16 @@ hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
     e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 1, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((q_stats_bf16<D, 1, CAUSAL>), grid, block, smem, s, p);
-  } else {
+  } else if (pass == FHOG_PASS_B) {
     const int smem = 2 * 4 * tile;
     e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 2, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((q_stats_bf16<D, 2, CAUSAL>), grid, block, smem, s, p);
+  } else {
+    const int smem = 2 * 4 * tile;
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 5, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((q_stats_bf16<D, 5, CAUSAL>), grid, block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -175,7 +206,7 @@ bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
   if (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV) return launch_bf16_pc_pass(p, pass, s);
-  if (pass != FHOG_PASS_DD && pass != FHOG_PASS_B) return hipErrorInvalidValue;
+  if (pass != FHOG_PASS_DD && pass != FHOG_PASS_B && pass != FHOG_PASS_DD_B) return hipErrorInvalidValue;
   if (p.d == 128) return p.causal ? launch_stats_d<128, true>(p, pass, s) : launch_stats_d<128, false>(p, pass, s);
   return p.causal ? launch_stats_d<64, true>(p, pass, s) : launch_stats_d<64, false>(p, pass, s);
 }

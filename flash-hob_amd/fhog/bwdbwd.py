@@ -83,7 +83,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
         impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the bf16 MFMA kernels for
             bf16 tensors whose shape they support, the fp32-MFMA kernels otherwise.
         return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
-        only_pass: run a single pass (0..4) instead of all five; for tests and profiling.
+        only_pass: run a single pass (0..5, see fhog._lib.PASS_*) instead of the whole chain; for tests and profiling.
 
     Returns:
         dQ2, dK2, dV2, ddO shaped and typed like Q, K, V, O (+ ``(d, dd, b)`` if ``return_stats``).

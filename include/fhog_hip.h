@@ -52,6 +52,8 @@ extern "C" {
 #define FHOG_PASS_B 2      /* b_i  = sum_j dP'_ij P_ij                        (fhog/triton_bwdbwd.py:217-251) */
 #define FHOG_PASS_DQ_DDO 3 /* dQ2 = dS ddK + dS' K ; ddO = P ddV + ddP V      (fhog/triton_bwdbwd.py:257-313) */
 #define FHOG_PASS_DK_DV 4  /* dK2 = dS^T ddQ + dS'^T Q ; dV2 = ddP^T dO       (fhog/triton_bwdbwd.py:467-535) */
+#define FHOG_PASS_DD_B 5   /* passes 1 and 2 in one sweep: b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
+                              (same quantities as fhog/triton_bwdbwd.py:185-251, three recomputed products fewer) */
 
 /* kernel families (fhog_bwdbwd_args.impl) */
 #define FHOG_IMPL_AUTO 0   /* bf16 MFMA kernels when the shape allows, else the fp32-MFMA kernels */
@@ -105,7 +107,8 @@ int fhog_validate(const fhog_bwdbwd_args* args);
    FHOG_IMPL_BF16, or a negative FHOG_E_* code. Host-only. */
 int fhog_select_impl(const fhog_bwdbwd_args* args);
 
-/* All passes in order (d, dd, b, dQ2+ddO, dK2+dV2) on `hip_stream` (a hipStream_t).
+/* All passes in order (d, dd and b, dQ2+ddO, dK2+dV2) on `hip_stream` (a hipStream_t); dd and b come
+   from one fused sweep (FHOG_PASS_DD_B) in the bf16 family and from passes 1 and 2 in the fp32 family.
    Drop-in for the two launches + reduction of flash_bwdbwd (fhog/triton_bwdbwd.py:580-646). */
 int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
 

@@ -141,6 +141,30 @@ def test_bf16_family_small(shape, causal):
     assert max(e2.values()) < 1.5e-2, e2
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("d", [64, 128])
+def test_bf16_fused_statistics_match_separate_passes(d, causal):
+    """The fused dd+b sweep (pass id 5, what the whole chain runs) against passes 1 and 2 run on their own."""
+    from fhog import BwdBwdPlan
+    x = with_caches(make_case(3, 384, 384, d, torch.bfloat16, seed=12, grad_std=0.1), d ** -0.5, causal)
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], d ** -0.5,
+                      causal=causal, impl="bf16")
+    plan.ws.fill_(float("nan"))
+    for i in (0, 1, 2):
+        plan.run(only_pass=i)
+    torch.cuda.synchronize()
+    separate = plan.ws.clone()
+    plan.ws[plan.ws.numel() // 3:].fill_(float("nan"))
+    plan.run(only_pass=5)
+    torch.cuda.synchronize()
+    fused = plan.ws.view(3, -1)
+    separate = separate.view(3, -1)
+    assert torch.isfinite(fused).all()
+    assert torch.equal(fused[0], separate[0])
+    assert normalised_max_error(fused[1], separate[1]) < 1e-6      # same sums, same order
+    assert normalised_max_error(fused[2], separate[2]) < 1e-3      # dd_i * sum_j P dP taken out of the sum
+
+
 def test_bf16_auto_dispatch():
     from fhog import BwdBwdPlan
     x = with_caches(make_case(2, 256, 256, 64, torch.bfloat16, seed=6), 0.125, False)
