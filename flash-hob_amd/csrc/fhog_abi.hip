@@ -30,6 +30,8 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
   if (a->impl != FHOG_IMPL_AUTO && a->impl != FHOG_IMPL_FP32 && a->impl != FHOG_IMPL_BF16)
     return fail(FHOG_E_DTYPE, "unknown impl %d", a->impl);
+  if (a->schedule != FHOG_SCHEDULE_FOUR_PASS && a->schedule != FHOG_SCHEDULE_FUSED_STATS)
+    return fail(FHOG_E_DTYPE, "unknown schedule %d", a->schedule);
   if (a->batch < 1 || a->n_q < 1 || a->n_k < 1)
     return fail(FHOG_E_SHAPE, "batch, n_q, n_k must be >= 1 (got %lld, %lld, %lld)", (long long)a->batch, (long long)a->n_q,
                 (long long)a->n_k);
@@ -145,9 +147,13 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   if (rc != FHOG_OK) return rc;
   const fhog::Params p = to_params(args);
   const int impl = select_impl(args);
-  const int order[] = {FHOG_PASS_D, FHOG_PASS_DD_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
-  for (int pass : order) {
-    const int r = run_pass(args, p, impl, pass, (hipStream_t)hip_stream);
+  const int four[] = {FHOG_PASS_D, FHOG_PASS_DD, FHOG_PASS_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
+  const int fused[] = {FHOG_PASS_D, FHOG_PASS_DD_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
+  const bool is_fused = args->schedule == FHOG_SCHEDULE_FUSED_STATS;
+  const int* order = is_fused ? fused : four;
+  const int n_pass = is_fused ? 4 : 5;
+  for (int i = 0; i < n_pass; i++) {
+    const int r = run_pass(args, p, impl, order[i], (hipStream_t)hip_stream);
     if (r != FHOG_OK) return r;
   }
   return FHOG_OK;

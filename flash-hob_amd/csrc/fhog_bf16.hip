@@ -51,6 +51,10 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   const float dsum = PASS != 1 ? p.ws_d[row] : 0.f;
   const float dd = PASS == 2 ? p.ws_dd[row] : 0.f;
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
+  // All register loads land here. The staging loads below are issued from inline asm, which the compiler's
+  // wait-count bookkeeping does not see: without this explicit wait it would keep "vmcnt(n)" waits for the
+  // resident operands inside the loop, where they would stall every iteration on the tile being staged.
+  wait_vm0();
 
   int aoff[KK];
 #pragma unroll

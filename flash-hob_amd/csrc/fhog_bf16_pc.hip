@@ -410,14 +410,15 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     dma.init(p.stride_qn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
     float stat_reg = 0.f;  // consumer threads 0..127: one statistic value of the staged tile
+    // A global (not generic) load, so that it does not tie up the LDS wait counter; issued before the staging
+    // loads of the step, so that reusing its destination register never waits for those.
+    // The loaded value is first touched in store_stat, at the end of the step: a use right after the load would
+    // make the wave wait there for the load and, with it, for every staging load issued before it.
     auto load_stat = [&](int q_base) {
-      if (ctid < 4 * TS) {
-        const float v = stat_src[ctid / TS][q_base + (ctid % TS)];
-        stat_reg = (ctid < TS) ? v * kLog2e : v;
-      }
+      if (ctid < 4 * TS) stat_reg = *(global_f32_ptr)(stat_src[ctid / TS] + q_base + (ctid % TS));
     };
     auto store_stat = [&](char* stage_base) {
-      if (ctid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * SM::TILE)[ctid] = stat_reg;
+      if (ctid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * SM::TILE)[ctid] = (ctid < TS) ? stat_reg * kLog2e : stat_reg;
     };
     {
       const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
@@ -433,9 +434,9 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       if (j + 1 < t_end) {
         const uint32_t dst = ring_lds + sn * SM::STAGE;
         const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
+        load_stat((j + 1) * TS);
 #pragma unroll
         for (int x = 0; x < 3; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
-        load_stat((j + 1) * TS);
       }
       if (j > t_begin && (!CAUSAL || (j - 1) * TS >= kw)) {
         const char* stage = smem + sc * SM::STAGE;

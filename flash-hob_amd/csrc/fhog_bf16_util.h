@@ -104,6 +104,10 @@ struct Dma {
   }
 };
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// s_waitcnt vmcnt(0) as a builtin (gfx9 encoding: vmcnt 0, expcnt 7, lgkmcnt 15), which the compiler's wait-count
+// pass takes into account: register loads issued before it are known to have landed.
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+typedef const __attribute__((address_space(1))) float* global_f32_ptr;
 __device__ __forceinline__ uint32_t lds_addr(const char* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }

@@ -31,7 +31,7 @@ class BwdBwdArgs(Structure):
         ("dq2", c_void_p), ("dk2", c_void_p), ("dv2", c_void_p), ("ddo", c_void_p), ("ws", c_void_p),
         ("batch", c_int64), ("n_q", c_int64), ("n_k", c_int64), ("d", c_int64),
         ("stride_qb", c_int64), ("stride_qn", c_int64), ("stride_kb", c_int64), ("stride_kn", c_int64),
-        ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("impl", c_int32), ("reserved", c_int32),
+        ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("impl", c_int32), ("schedule", c_int32),
     ]
 
 

@@ -44,7 +44,7 @@ def workspace_floats(batch: int, n_q: int) -> int:
     return _lib.lib().fhog_bwdbwd_workspace_bytes(batch, n_q) // 4
 
 
-def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws) -> _lib.BwdBwdArgs:
+def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, fused_stats=False) -> _lib.BwdBwdArgs:
     a = _lib.BwdBwdArgs()
     a.q, a.k, a.v, a.o, a.dO = Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dO.data_ptr()
     a.ddq, a.ddk, a.ddv = ddQ.data_ptr(), ddK.data_ptr(), ddV.data_ptr()
@@ -59,11 +59,12 @@ def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws)
     a.dtype = _DTYPES[Q.dtype]
     a.causal = int(bool(causal))
     a.impl = impl
+    a.schedule = 1 if fused_stats else 0
     return a
 
 
 def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = False, impl: Optional[str] = None,
-                 return_stats: bool = False, only_pass: Optional[int] = None):
+                 fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None):
     """Flash Higher-Order-Gradients: VJP of the attention backward pass.
 
     Same positional signature and return order as the reference
@@ -82,6 +83,9 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
             double-backward.)
         impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the bf16 MFMA kernels for
             bf16 tensors whose shape they support, the fp32-MFMA kernels otherwise.
+        fused_stats: opt-in schedule that takes ``dd`` and ``b`` from one sweep instead of the reference's two
+            (``fhog/triton_bwdbwd.py:185-251``): 22 instead of 25 recomputed products; ``b`` then differs from the
+            default schedule's value only by fp32 summation order.
         return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
         only_pass: run a single pass (0..5, see fhog._lib.PASS_*) instead of the whole chain; for tests and profiling.
 
@@ -137,7 +141,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
         dv2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
         ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
         args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl],
-                           (dq2, dk2, dv2, ddo), ws)
+                           (dq2, dk2, dv2, ddo), ws, fused_stats)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         L_ = _lib.lib()
         if only_pass is None:
@@ -160,7 +164,7 @@ class BwdBwdPlan:
     For benchmark loops and per-pass profiling; ``flash_bwdbwd`` is the drop-in entry point.
     """
 
-    def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, impl=None):
+    def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, impl=None, fused_stats=False):
         ts = [_flatten(t, "tensor") for t in (Q, K, V, O, dO, ddQ, ddK, ddV)]
         q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = ts
         q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
@@ -170,7 +174,7 @@ class BwdBwdPlan:
         self.keep = (q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse)
         self.outs = (torch.empty_like(q3), torch.empty_like(k3), torch.empty_like(v3), torch.empty_like(q3))
         self.ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
-        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws)
+        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws, fused_stats)
         self.lib = _lib.lib()
         _lib.check(self.lib.fhog_validate(ctypes.byref(self.args)))
         self.impl = self.lib.fhog_select_impl(ctypes.byref(self.args))

@@ -48,9 +48,9 @@ class Workload:
 
     @property
     def flops_executed(self) -> int:
-        """22 contractions issued by the bf16 family: fused dd+b sweep 5, dQ'+ddO sweep 9, dK'+dV' sweep 8
-        (the fp32 family runs dd and b as separate sweeps: 3 + 5 + 9 + 8 = 25)."""
-        return 44 * self.d * self.pairs
+        """25 contractions issued by the four recomputation passes (3 + 5 + 9 + 8); the opt-in fused
+        statistics sweep issues 22 (5 + 9 + 8)."""
+        return 50 * self.d * self.pairs
 
     @property
     def bytes_algorithmic(self) -> int:

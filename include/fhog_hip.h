@@ -60,6 +60,12 @@ extern "C" {
 #define FHOG_IMPL_FP32 1   /* force the fp32-MFMA kernels (any dtype; every intermediate in fp32) */
 #define FHOG_IMPL_BF16 2   /* force the bf16 MFMA kernels; error if the shape/dtype does not fit */
 
+/* pass schedules of fhog_bwdbwd (fhog_bwdbwd_args.schedule) */
+#define FHOG_SCHEDULE_FOUR_PASS 0   /* the reference's schedule: d, then dd, b, dQ2+ddO, dK2+dV2 as four sweeps
+                                       (fhog/triton_bwdbwd.py:185-313, 467-535); 25 recomputed products */
+#define FHOG_SCHEDULE_FUSED_STATS 1 /* opt-in: dd and b from one sweep (FHOG_PASS_DD_B), 22 recomputed products;
+                                       b differs from the four-pass value only by fp32 summation order */
+
 typedef struct fhog_bwdbwd_args {
   /* inputs (device pointers); q, o, dO, ddq: (batch, n_q, d); k, v, ddk, ddv: (batch, n_k, d) */
   const void* q;
@@ -86,7 +92,7 @@ typedef struct fhog_bwdbwd_args {
   int32_t dtype;  /* FHOG_DTYPE_* */
   int32_t causal; /* 0 | 1 (top-left mask: key j visible to query i iff j <= i; needs n_q == n_k) */
   int32_t impl;   /* FHOG_IMPL_* */
-  int32_t reserved;
+  int32_t schedule; /* FHOG_SCHEDULE_* */
 } fhog_bwdbwd_args;
 
 /* Version of this header the library was built from. */
@@ -107,8 +113,8 @@ int fhog_validate(const fhog_bwdbwd_args* args);
    FHOG_IMPL_BF16, or a negative FHOG_E_* code. Host-only. */
 int fhog_select_impl(const fhog_bwdbwd_args* args);
 
-/* All passes in order (d, dd and b, dQ2+ddO, dK2+dV2) on `hip_stream` (a hipStream_t); dd and b come
-   from one fused sweep (FHOG_PASS_DD_B) in the bf16 family and from passes 1 and 2 in the fp32 family.
+/* All passes in order (d, dd, b, dQ2+ddO, dK2+dV2) on `hip_stream` (a hipStream_t); with
+   schedule = FHOG_SCHEDULE_FUSED_STATS, dd and b come from one sweep (FHOG_PASS_DD_B) instead.
    Drop-in for the two launches + reduction of flash_bwdbwd (fhog/triton_bwdbwd.py:580-646). */
 int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
 

@@ -121,15 +121,17 @@ def test_strided_and_4d_inputs():
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("shape", [(2, 128, 128, 64), (3, 256, 256, 128), (2, 128, 384, 64), (9, 384, 128, 128),
                                    (1, 512, 512, 128)])
-def test_bf16_family_small(shape, causal):
-    """bf16 MFMA kernels against the fp64 closed form, including the row vectors of passes 0..2."""
+@pytest.mark.parametrize("fused_stats", [False, True])
+def test_bf16_family_small(shape, causal, fused_stats):
+    """bf16 MFMA kernels against the fp64 closed form, including the row vectors of passes 0..2, under the
+    four-pass schedule and the opt-in fused statistics sweep."""
     batch, n_q, n_k, d = shape
     if causal:
         n_k = n_q
     x = make_case(batch, n_q, n_k, d, torch.bfloat16, seed=5, grad_std=0.1)
     scale = d ** -0.5
     x = with_caches(x, scale, causal)
-    outs = run_fhog(x, scale, causal, impl="bf16", return_stats=True)
+    outs = run_fhog(x, scale, causal, impl="bf16", return_stats=True, fused_stats=fused_stats)
     ref = reference_fp64_cpu(x, scale, causal)
     e = errors(outs[:4], [ref[n] for n in NAMES])
     assert max(e.values()) < 2e-2, e
@@ -175,13 +177,13 @@ def test_bf16_auto_dispatch():
     assert plan.impl == 1
 
 
-def _full_config(name, seed, heads=None):
+def _full_config(name, seed, heads=None, fused_stats=False):
     from fhog.workloads import WORKLOADS, make_inputs
     w = WORKLOADS[name]
     x = make_inputs(w, seed, device="cuda:0")
     x = {n: t.flatten(0, 1) for n, t in x.items()}
     x = with_caches(x, w.scale, w.causal)
-    outs = run_fhog(x, w.scale, w.causal)
+    outs = run_fhog(x, w.scale, w.causal, fused_stats=fused_stats)
     hs = list(range(w.batch)) if heads is None else heads
     worst = {}
     for h0 in range(0, len(hs), 4):
@@ -203,6 +205,11 @@ def test_cfg1_bf16_noncausal_2048_d64(seed):
 @pytest.mark.parametrize("seed", [0, 1])
 def test_cfg2_bf16_causal_4096_d128_headline(seed):
     w, e = _full_config("cfg2_bf16_causal_4096_d128", seed)
+    assert max(e.values()) < 2e-2, e
+
+
+def test_cfg2_headline_fused_statistics_schedule():
+    w, e = _full_config("cfg2_bf16_causal_4096_d128", 2, fused_stats=True)
     assert max(e.values()) < 2e-2, e
 
 
