@@ -87,7 +87,7 @@ def main():
 
     x_cpu = {n: t.flatten(0, 1) for n, t in make_inputs(w, seed=0).items()}
     x = {n: t.to(dev) for n, t in x_cpu.items()}
-    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)   # caches; not timed
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal, use_hip=False)   # caches (fp32 forward); not timed
     call = lambda: fhog.flash_bwdbwd(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale,
                                      causal=w.causal)
     plan = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale, causal=w.causal)

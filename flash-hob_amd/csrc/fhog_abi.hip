@@ -113,9 +113,92 @@ int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& p, int impl, int pas
   return FHOG_OK;
 }
 
+int validate_attn(const fhog_attn_args* a, int backward) {
+  if (!a) return fail(FHOG_E_NULL, "args is NULL");
+  const void* ptrs[] = {a->q, a->k, a->v, a->o, a->lse, a->dO, a->dq, a->dk, a->dv, a->ws};
+  const char* names[] = {"q", "k", "v", "o", "lse", "dO", "dq", "dk", "dv", "ws"};
+  const int n_ptr = backward ? 10 : 5;
+  for (int i = 0; i < n_ptr; i++) {
+    if (!ptrs[i]) return fail(FHOG_E_NULL, "pointer '%s' is NULL", names[i]);
+    if (!aligned16(ptrs[i])) return fail(FHOG_E_ALIGN, "pointer '%s' is not 16-byte aligned", names[i]);
+  }
+  if (a->dtype != FHOG_DTYPE_BF16) return fail(FHOG_E_DTYPE, "the first-order kernels take bf16 tensors (dtype %d given)", a->dtype);
+  if (a->batch < 1 || a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld outside 1..65535", (long long)a->batch);
+  if (a->n_q < 1 || a->n_k < 1 || a->n_q > (1 << 24) || a->n_k > (1 << 24) || a->batch * a->n_q >= (int64_t)1 << 31)
+    return fail(FHOG_E_SHAPE, "n_q/n_k out of range");
+  if (a->causal != 0 && a->causal != 1) return fail(FHOG_E_CAUSAL, "causal must be 0 or 1");
+  if (a->causal && a->n_q != a->n_k) return fail(FHOG_E_CAUSAL, "causal needs n_q == n_k");
+  if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
+    return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128} and n_q, n_k multiples of 128");
+  if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
+  if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
+  if (a->stride_qn % 8 || a->stride_kn % 8 || a->stride_qb % 8 || a->stride_kb % 8)
+    return fail(FHOG_E_STRIDE, "strides must be multiples of 8 elements (16 bytes)");
+  if (a->batch > 1 && (a->stride_qb < a->n_q * a->stride_qn || a->stride_kb < a->n_k * a->stride_kn))
+    return fail(FHOG_E_STRIDE, "batch stride smaller than one (n, d) slice");
+  return FHOG_OK;
+}
+
+fhog::AttnParams to_attn_params(const fhog_attn_args* a) {
+  fhog::AttnParams p;
+  p.q = a->q;
+  p.k = a->k;
+  p.v = a->v;
+  p.o = a->o;
+  p.lse = a->lse;
+  p.dO = a->dO;
+  p.dq = a->dq;
+  p.dk = a->dk;
+  p.dv = a->dv;
+  p.ws_d = a->ws;
+  p.stride_qb = a->stride_qb;
+  p.stride_qn = a->stride_qn;
+  p.stride_kb = a->stride_kb;
+  p.stride_kn = a->stride_kn;
+  p.batch = (int32_t)a->batch;
+  p.n_q = (int32_t)a->n_q;
+  p.n_k = (int32_t)a->n_k;
+  p.d = (int32_t)a->d;
+  p.scale = a->scale;
+  p.causal = a->causal;
+  return p;
+}
+
 }  // namespace
 
 extern "C" {
+
+size_t fhog_attn_args_size(void) { return sizeof(fhog_attn_args); }
+
+int fhog_attn_validate(const fhog_attn_args* args, int backward) { return validate_attn(args, backward); }
+
+int fhog_attn_fwd(const fhog_attn_args* args, void* hip_stream) {
+  const int rc = validate_attn(args, 0);
+  if (rc != FHOG_OK) return rc;
+  const hipError_t e = fhog::launch_attn_bf16(to_attn_params(args), 0, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "attention forward: HIP error %d (%s)", (int)e, hipGetErrorString(e));
+  return FHOG_OK;
+}
+
+int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream) {
+  const int rc = validate_attn(args, 1);
+  if (rc != FHOG_OK) return rc;
+  const fhog::AttnParams p = to_attn_params(args);
+  fhog::Params rd = {};  // row sums d_i = sum_c o_ic dO_ic with the kernel of pass 0
+  rd.o = args->o;
+  rd.dO = args->dO;
+  rd.ws_d = args->ws;
+  rd.stride_qb = p.stride_qb;
+  rd.stride_qn = p.stride_qn;
+  rd.batch = p.batch;
+  rd.n_q = p.n_q;
+  rd.d = p.d;
+  hipError_t e = fhog::launch_rowdot(rd, FHOG_DTYPE_BF16, (hipStream_t)hip_stream);
+  for (int which = 1; which <= 2 && e == hipSuccess; which++) e = fhog::launch_attn_bf16(p, which, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "attention backward: HIP error %d (%s)", (int)e, hipGetErrorString(e));
+  return FHOG_OK;
+}
+
 
 int fhog_abi_version(void) { return FHOG_ABI_VERSION; }
 

@@ -1,0 +1,432 @@
+// First-order attention on gfx950 bf16 MFMA: the callers on either side of the double-backward.
+//   attn_fwd_bf16     O and fp32 L = logsumexp        (fhog/triton_flash.py:12-133; L also replaces produce_L, :252-258)
+//   attn_bwd_q_bf16   dQ                 Q-tiled      (fhog/triton_flash.py:201-220: P, dP, dS, dQ)
+//   attn_bwd_k_bf16   dK, dV             K-tiled      (fhog/triton_flash.py:201-220: dV, dK)
+// No atomics and nothing of shape (N_Q, N_K) in memory: like the double-backward, the backward recomputes
+// S and dP once per tiling direction.
+//
+// A workgroup is 256 threads = 4 wave64 owning 128 stationary rows (queries, or keys in the K-tiled kernel);
+// tiles of 32 streamed rows go through a two-stage LDS ring filled by direct global->LDS loads. First-level
+// products are computed transposed (streamed rows = M, stationary rows = N), so a lane owns ONE stationary row
+// and the soft-max statistics are per-lane scalars. The accumulator layout of such a product (lane = column,
+// registers = streamed rows 8g + 4h + j) is, after rounding to bf16, already a valid B operand of the
+// second-level MFMA whose contraction runs over the streamed rows: slot e of k-step t stands for streamed row
+// 16t + 8(e/4) + 4h + e%4, and the A operand (the transposed value tile) is fetched from LDS with transposing
+// reads that use the same row order. Second-level operands therefore never pass through LDS.
+#include "fhog_bf16_util.h"
+
+namespace fhog {
+using namespace bf16k;
+namespace {
+
+// Transposed A operand for a B operand that is an S-shaped accumulator kept in registers: lane
+// (col = lane%32, h = lane/32) of 32-column block cb receives, for k-step t, tile rows 16t + 4h + 0..3 (first
+// read) and 16t + 8 + 4h + 0..3 (second read) at column cb*32 + col. Per-lane part of the address, s = 0 | 1.
+template <int D>
+__device__ __forceinline__ int tr_lane_off_acc(int cb, int s, int lane) {
+  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
+  const int col = cb * 32 + 16 * b + 4 * (i & 3);
+  const int r = 8 * s + 4 * h + (i >> 2);
+  return tile_off<D>(r, col >> 3) + ((col >> 2) & 1) * 8;
+}
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+// registers 8t .. 8t+7 of an S-shaped fp32 tile as the bf16 B operand of second-level k-step t
+__device__ __forceinline__ bf16x8_t pack_operand(const f32x16_t& x, int t) {
+  u32x4_t u = {pack2(x[8 * t + 0], x[8 * t + 1]), pack2(x[8 * t + 2], x[8 * t + 3]), pack2(x[8 * t + 4], x[8 * t + 5]),
+               pack2(x[8 * t + 6], x[8 * t + 7])};
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
+// acc[cb] += tile^T (columns 32cb..32cb+31) x operand, for both k-steps and all column blocks of the tile
+template <int D, int NOP>
+__device__ __forceinline__ void second_level(const char* const (&tile)[NOP], const int (&troff)[D / 32][2],
+                                             const bf16x8_t (&op)[NOP][2], f32x16_t (&acc)[NOP][D / 32]) {
+  constexpr int NC = D / 32, NIT = 2 * NC;
+  bf16x8_t a[2][NOP];
+#pragma unroll
+  for (int x = 0; x < NOP; x++) a[0][x] = lds_read_tr_pre(tile[x] + troff[0][0], tile[x] + troff[0][1], 0);
+#pragma unroll
+  for (int it = 0; it < NIT; it++) {
+    const int t = it / NC, cb = it % NC, c = it & 1;
+    if (it + 1 < NIT) {
+      const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+#pragma unroll
+      for (int x = 0; x < NOP; x++)
+        a[c ^ 1][x] = lds_read_tr_pre(tile[x] + troff[cb1][0], tile[x] + troff[cb1][1], t1 * 16 * 2 * D);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int x = 0; x < NOP; x++) acc[x][cb] = mfma(a[c][x], op[x][t], acc[x][cb]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// first-level product of one streamed tile with resident rows: out += tile x res^T (streamed rows = M)
+template <int D, int NRES>
+__device__ __forceinline__ void first_level(const char* tile, const int (&aoff)[D / 16], const bf16x8_t* const (&res)[NRES],
+                                            f32x16_t (&out)[NRES]) {
+  constexpr int KK = D / 16, PF = 2, NB = PF + 1;
+  bf16x8_t a[NB];
+#pragma unroll
+  for (int i = 0; i < PF; i++) a[i] = lds_read128(tile, aoff[i]);
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+    if (kk + PF < KK) a[(kk + PF) % NB] = lds_read128(tile, aoff[kk + PF]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int x = 0; x < NRES; x++) out[x] = mfma(a[kk % NB], res[x][kk], out[x]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// ---- forward -----------------------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
+
+  int bh, tile;
+  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[2] = {(const __bf16*)p.k + koff, (const __bf16*)p.v + koff};
+
+  bf16x8_t Qb[KK];
+  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
+  wait_vm0();
+  const float c_scale_log2 = p.scale * kLog2e;
+
+  int aoff[KK], troff[NC][2];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  float m = -INFINITY, l = 0.f;  // running maximum (log2 units) of the row; this lane's half of the row sum
+  f32x16_t acc[1][NC];           // O^T: acc[0][cb][r] = (column 32cb + 8(r/4) + 4h + r%4, query qi)
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
+
+  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  Dma<D> dma;
+  dma.init(p.stride_kn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+#pragma unroll
+  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave);
+  dma_wait();
+  __syncthreads();
+
+  for (int j = 0; j < n_tiles; j++) {
+    if (j + 1 < n_tiles) {
+      const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
+      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
+#pragma unroll
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+    }
+    const int k0 = j * TS;
+    if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
+      const char* stage = smem + (j & 1) * STAGE;
+      f32x16_t s[1] = {f32x16_t{0}};
+      const bf16x8_t* const res[1] = {Qb};
+      first_level<D, 1>(stage, aoff, res, s);  // S^T: s[r] = (key k0 + 8(r/4) + 4h + r%4, query qi)
+      f32x16_t x;
+#pragma unroll
+      for (int r = 0; r < 16; r++) x[r] = s[0][r] * c_scale_log2;
+      if (CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
+        const int lim = qi - k0 - 4 * h;
+#pragma unroll
+        for (int r = 0; r < 16; r++) x[r] = (8 * (r / 4) + (r % 4) <= lim) ? x[r] : -INFINITY;
+      }
+      float tmax = x[0];
+#pragma unroll
+      for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, x[r]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      const float m_new = fmaxf(m, tmax);  // finite: key 0 is visible to every query and tiles come in key order
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      float rs = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+        rs += x[r];
+      }
+      l = __builtin_fmaf(l, alpha, rs);
+      if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // rescale only when some row's maximum moved
+#pragma unroll
+        for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[0][cb][r] *= alpha;
+      }
+      m = m_new;
+      const bf16x8_t op[1][2] = {{pack_operand(x, 0), pack_operand(x, 1)}};
+      const char* const vt[1] = {stage + TILE};
+      second_level<D, 1>(vt, troff, op, acc);  // O^T += V^T P^T
+    }
+    dma_wait();
+    __syncthreads();
+  }
+  l += __shfl_xor(l, 32);
+  const float inv = 1.f / l;
+  __bf16* o = (__bf16*)p.o + qoff + (int64_t)qi * p.stride_qn;
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      bf16x4_t v;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = (__bf16)(acc[0][cb][4 * g + e] * inv);
+      *reinterpret_cast<bf16x4_t*>(o + 32 * cb + 8 * g + 4 * h) = v;
+    }
+  if (h == 0) p.lse[(int64_t)bh * p.n_q + qi] = (m + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;  // v_log_f32 is log2
+}
+
+// ---- backward, Q-tiled: dQ -----------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
+
+  int bh, tile;
+  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[2] = {(const __bf16*)p.k + koff, (const __bf16*)p.v + koff};
+
+  bf16x8_t Qb[KK], dOb[KK];
+  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
+  load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
+  const int64_t row = (int64_t)bh * p.n_q + qi;
+  const float l_log2 = p.lse[row] * kLog2e, dsum = p.ws_d[row];
+  wait_vm0();
+  const float c_scale_log2 = p.scale * kLog2e;
+
+  int aoff[KK], troff[NC][2];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  f32x16_t acc[1][NC];  // dQ^T
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
+
+  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  Dma<D> dma;
+  dma.init(p.stride_kn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+#pragma unroll
+  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave);
+  dma_wait();
+  __syncthreads();
+
+  for (int j = 0; j < n_tiles; j++) {
+    if (j + 1 < n_tiles) {
+      const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
+      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
+#pragma unroll
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+    }
+    const int k0 = j * TS;
+    if (!CAUSAL || k0 <= qw) {
+      const char* stage = smem + (j & 1) * STAGE;
+      f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
+      const bf16x8_t* const rq[1] = {Qb};
+      const bf16x8_t* const rdo[1] = {dOb};
+      first_level<D, 1>(stage, aoff, rq, s);           // S^T  = K Q^T
+      first_level<D, 1>(stage + TILE, aoff, rdo, dp);  // dP^T = V dO^T
+      f32x16_t ds;
+#pragma unroll
+      for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * (dp[0][r] - dsum);
+      if (CAUSAL && k0 == qw) {
+        const int lim = qi - k0 - 4 * h;
+#pragma unroll
+        for (int r = 0; r < 16; r++) ds[r] = (8 * (r / 4) + (r % 4) <= lim) ? ds[r] : 0.f;
+      }
+      const bf16x8_t op[1][2] = {{pack_operand(ds, 0), pack_operand(ds, 1)}};
+      const char* const kt[1] = {stage};
+      second_level<D, 1>(kt, troff, op, acc);  // dQ^T += K^T dS^T
+    }
+    dma_wait();
+    __syncthreads();
+  }
+  __bf16* o = (__bf16*)p.dq + qoff + (int64_t)qi * p.stride_qn;
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      bf16x4_t v;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = (__bf16)(acc[0][cb][4 * g + e] * p.scale);
+      *reinterpret_cast<bf16x4_t*>(o + 32 * cb + 8 * g + 4 * h) = v;
+    }
+}
+
+// ---- backward, K-tiled: dK, dV ---------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
+  constexpr int STAT = 2 * TS * 4;         // L log2(e) and d of the 32 staged queries
+  constexpr int STAGE = 2 * TILE + STAT;   // Q tile, dO tile, statistics
+
+  int bh, tile;
+  if (!decode_block(p.n_k / WG_ROWS, p.batch, false, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int k0 = tile * WG_ROWS, kw = k0 + 32 * wave, kj = kw + n;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[2] = {(const __bf16*)p.q + qoff, (const __bf16*)p.dO + qoff};
+  const float* stat_src = (tid < TS ? p.lse : p.ws_d) + (int64_t)bh * p.n_q + (tid & (TS - 1));
+
+  bf16x8_t Kb[KK], Vb[KK];
+  load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kj, h);
+  load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kj, h);
+  const float c_scale_log2 = p.scale * kLog2e;
+
+  int aoff[KK], troff[NC][2];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  f32x16_t acc[2][NC];  // [0]: dK^T, [1]: dV^T
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    acc[0][cb] = f32x16_t{0};
+    acc[1][cb] = f32x16_t{0};
+  }
+  // causal: query tiles before this workgroup's first key see none of its keys
+  const int t_begin = CAUSAL ? k0 / TS : 0, t_end = p.n_q / TS;
+  Dma<D> dma;
+  dma.init(p.stride_qn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  float stat_reg = 0.f;  // threads 0..63: one statistic of the tile being staged
+  // The statistic is loaded before the staging loads of a step and first touched at the end of the step, so the
+  // wave never waits for it in between.
+  auto load_stat = [&](int q_base) {
+    if (tid < 2 * TS) stat_reg = *(global_f32_ptr)(stat_src + q_base);
+  };
+  auto store_stat = [&](char* stage_base) {
+    if (tid < 2 * TS) reinterpret_cast<float*>(stage_base + 2 * TILE)[tid] = (tid < TS) ? stat_reg * kLog2e : stat_reg;
+  };
+  {
+    load_stat(t_begin * TS);
+    const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
+#pragma unroll
+    for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x] + adv, wave);
+    wait_vm0();
+    store_stat(smem);
+  }
+  __syncthreads();
+
+  for (int j = t_begin; j < t_end; j++) {
+    const int st = (j - t_begin) & 1;
+    if (j + 1 < t_end) {
+      load_stat((j + 1) * TS);
+      const uint32_t dst = ring_lds + (st ^ 1) * STAGE;
+      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
+#pragma unroll
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+    }
+    const int qb = j * TS;
+    if (!CAUSAL || qb >= kw) {  // else no query of the tile sees a key of this wave
+      const char* stage = smem + st * STAGE;
+      const float* stat = reinterpret_cast<const float*>(stage + 2 * TILE);
+      f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
+      const bf16x8_t* const rk[1] = {Kb};
+      const bf16x8_t* const rv[1] = {Vb};
+      first_level<D, 1>(stage, aoff, rk, s);           // S  = Q K^T : s[r] = (query qb + 8(r/4) + 4h + r%4, key kj)
+      first_level<D, 1>(stage + TILE, aoff, rv, dp);   // dP = dO V^T
+      f32x16_t pv, ds;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 8 * g + 4 * h);
+        const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(stat + TS + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = 4 * g + e;
+          pv[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l4[e]);
+          ds[r] = dp[0][r] - d4[e];
+        }
+      }
+      if (CAUSAL && qb == kw) {  // wave-uniform: only the block on the diagonal
+        const int lim = kj - qb - 4 * h;  // query row 8g + 4h + e sees key kj iff 8g + e >= lim
+#pragma unroll
+        for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) >= lim) ? pv[r] : 0.f;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) ds[r] *= pv[r];
+      const bf16x8_t op[2][2] = {{pack_operand(ds, 0), pack_operand(ds, 1)}, {pack_operand(pv, 0), pack_operand(pv, 1)}};
+      const char* const tl[2] = {stage, stage + TILE};
+      second_level<D, 2>(tl, troff, op, acc);  // dK^T += Q^T dS ; dV^T += dO^T P
+    }
+    if (j + 1 < t_end) {
+      wait_vm0();
+      store_stat(smem + (st ^ 1) * STAGE);
+    }
+    dma_wait();
+    __syncthreads();
+  }
+  __bf16* odk = (__bf16*)p.dk + koff + (int64_t)kj * p.stride_kn;
+  __bf16* odv = (__bf16*)p.dv + koff + (int64_t)kj * p.stride_kn;
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      bf16x4_t a, b;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        a[e] = (__bf16)(acc[0][cb][4 * g + e] * p.scale);
+        b[e] = (__bf16)acc[1][cb][4 * g + e];
+      }
+      *reinterpret_cast<bf16x4_t*>(odk + 32 * cb + 8 * g + 4 * h) = a;
+      *reinterpret_cast<bf16x4_t*>(odv + 32 * cb + 8 * g + 4 * h) = b;
+    }
+}
+
+template <typename K>
+hipError_t launch(K kernel, unsigned grid, int smem, hipStream_t s, const AttnParams& p) {
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, s, p);
+  return hipGetLastError();
+}
+
+template <int D, bool CAUSAL>
+hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
+  const unsigned heads8 = (unsigned)((p.batch + 7) / 8 * 8);
+  constexpr int TILE = TS * 2 * D;
+  switch (which) {
+    case 0: return launch(attn_fwd_bf16<D, CAUSAL>, heads8 * (p.n_q / WG_ROWS), 2 * 2 * TILE, s, p);
+    case 1: return launch(attn_bwd_q_bf16<D, CAUSAL>, heads8 * (p.n_q / WG_ROWS), 2 * 2 * TILE, s, p);
+    default: return launch(attn_bwd_k_bf16<D, CAUSAL>, heads8 * (p.n_k / WG_ROWS), 2 * (2 * TILE + 2 * TS * 4), s, p);
+  }
+}
+
+}  // namespace
+
+// which: 0 forward, 1 backward Q-tiled (dQ), 2 backward K-tiled (dK, dV)
+hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s) {
+  if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
+  if (p.d == 128) return p.causal ? launch_attn_d<128, true>(p, which, s) : launch_attn_d<128, false>(p, which, s);
+  return p.causal ? launch_attn_d<64, true>(p, which, s) : launch_attn_d<64, false>(p, which, s);
+}
+
+}  // namespace fhog

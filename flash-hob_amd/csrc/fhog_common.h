@@ -41,10 +41,29 @@ struct Params {
   int32_t causal;
 };
 
+// Kernel-side view of fhog_attn_args (first-order forward and backward).
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;        // forward: written; backward: read
+  float* lse;     // forward: written; backward: read
+  const void* dO; // backward only
+  void* dq;
+  void* dk;
+  void* dv;
+  float* ws_d;    // backward: (batch, n_q) row sums of O * dO
+  int64_t stride_qb, stride_qn, stride_kb, stride_kn;
+  int32_t batch, n_q, n_k, d;
+  float scale;
+  int32_t causal;
+};
+
 // Launchers implemented in the kernel translation units. Each returns hipGetLastError().
 hipError_t launch_rowdot(const Params& p, int dtype, hipStream_t s);                 // pass 0
 hipError_t launch_fp32_pass(const Params& p, int dtype, int pass, hipStream_t s);   // passes 1..4, fp32 MFMA
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s);              // passes 1..4, bf16 MFMA
+hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s);         // 0 forward, 1 dQ, 2 dK and dV
 bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal);
 
 }  // namespace fhog

@@ -35,6 +35,17 @@ class BwdBwdArgs(Structure):
     ]
 
 
+class AttnArgs(Structure):
+    """Mirror of ``fhog_attn_args``."""
+    _fields_ = [
+        ("q", c_void_p), ("k", c_void_p), ("v", c_void_p), ("o", c_void_p), ("lse", c_void_p),
+        ("dO", c_void_p), ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p), ("ws", c_void_p),
+        ("batch", c_int64), ("n_q", c_int64), ("n_k", c_int64), ("d", c_int64),
+        ("stride_qb", c_int64), ("stride_qn", c_int64), ("stride_kb", c_int64), ("stride_kn", c_int64),
+        ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("reserved", c_int32),
+    ]
+
+
 class FhogError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f"{ERROR_NAMES.get(code, code)}: {message}")
@@ -70,6 +81,16 @@ def lib() -> ctypes.CDLL:
     L.fhog_last_error.argtypes = []
     L.fhog_bwdbwd_args_size.restype = c_size_t
     L.fhog_bwdbwd_args_size.argtypes = []
+    L.fhog_attn_args_size.restype = c_size_t
+    L.fhog_attn_args_size.argtypes = []
+    L.fhog_attn_validate.restype = c_int
+    L.fhog_attn_validate.argtypes = [POINTER(AttnArgs), c_int]
+    L.fhog_attn_fwd.restype = c_int
+    L.fhog_attn_fwd.argtypes = [POINTER(AttnArgs), c_void_p]
+    L.fhog_attn_bwd.restype = c_int
+    L.fhog_attn_bwd.argtypes = [POINTER(AttnArgs), c_void_p]
+    if L.fhog_attn_args_size() != ctypes.sizeof(AttnArgs):
+        raise RuntimeError("fhog_attn_args layout differs between libfhog_hip.so and the ctypes mirror")
     if L.fhog_bwdbwd_args_size() != ctypes.sizeof(BwdBwdArgs):
         raise RuntimeError("fhog_bwdbwd_args layout differs between libfhog_hip.so and the ctypes mirror")
     if L.fhog_abi_version() != ABI_VERSION:

@@ -10,17 +10,22 @@ commented stub (``fhog/triton_bwdbwd.py:538-554``).  Here it is wired:
     AttnBwd.forward          -> dQ, dK, dV   (first-order backward)
     AttnBwd.backward         -> flash_bwdbwd(...) -> dQ', dK', dV', ddO
 
-The forward and the first-order backward are the callers on either side of the hot path;
-they are linear-memory torch compositions (blocked over heads and query rows, fp32
-accumulation), not tuned kernels.  The double-backward is the HIP library.
+The forward and the first-order backward are the callers on either side of the hot path.  For bf16
+tensors with d in {64, 128} and sequence lengths that are multiples of 128 they run as HIP kernels of
+the same library (``fhog_attn_fwd`` / ``fhog_attn_bwd``); every other dtype or shape takes
+linear-memory torch compositions on the GPU (blocked over heads and query rows, fp32 accumulation).
+The double-backward is always the HIP library.
 """
 from __future__ import annotations
 
 import math
 from typing import Optional, Tuple
 
+import ctypes
+
 import torch
 
+from . import _lib
 from .bwdbwd import flash_bwdbwd
 
 _BLOCK_ELEMS = 1 << 26  # fp32 elements of one materialised (heads, rows, N_K) block (256 MiB)
@@ -45,22 +50,94 @@ def _scores(q, k, scale, causal, r0):
     return s
 
 
-def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = False):
+def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
+    """Arguments for the HIP first-order kernels, or None when they do not cover these tensors."""
+    if not (q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == v.dtype == torch.bfloat16):
+        return None
+    a = _lib.AttnArgs()
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    a.batch, a.n_q, a.d = q.shape
+    a.n_k = k.shape[1]
+    a.stride_qb, a.stride_qn = q.stride(0), q.stride(1)
+    a.stride_kb, a.stride_kn = k.stride(0), k.stride(1)
+    a.scale, a.dtype, a.causal = float(scale), _lib.DTYPE_BF16, int(bool(causal))
+    return a
+
+
+def _same_layout(ts) -> bool:
+    return all(t.stride() == ts[0].stride() and t.stride(-1) == 1 for t in ts)
+
+
+def _attention_forward_hip(q, k, v, scale, causal):
+    """O and L from ``fhog_attn_fwd``; None when the kernels do not cover the arguments."""
+    q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
+    if not _same_layout([k, v]):
+        k, v = k.contiguous(), v.contiguous()
+    a = _hip_args(q, k, v, scale, causal)
+    if a is None:
+        return None
+    L_ = _lib.lib()
+    with torch.cuda.device(q.device):
+        o = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+        lse = torch.empty(q.shape[0], q.shape[1], dtype=torch.float32, device=q.device)
+        a.o, a.lse = o.data_ptr(), lse.data_ptr()
+        if L_.fhog_attn_validate(ctypes.byref(a), 0) != 0:
+            return None
+        _lib.check(L_.fhog_attn_fwd(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    return o, lse
+
+
+def _attention_backward_hip(q, k, v, o, do, L, scale, causal):
+    ts_q = [t if t.stride(-1) == 1 else t.contiguous() for t in (q, o, do)]
+    if not _same_layout(ts_q):
+        ts_q = [t.contiguous() for t in ts_q]
+    ts_k = [t if t.stride(-1) == 1 else t.contiguous() for t in (k, v)]
+    if not _same_layout(ts_k):
+        ts_k = [t.contiguous() for t in ts_k]
+    (q, o, do), (k, v) = ts_q, ts_k
+    a = _hip_args(q, k, v, scale, causal)
+    if a is None or o.dtype != torch.bfloat16 or do.dtype != torch.bfloat16:
+        return None
+    L_ = _lib.lib()
+    with torch.cuda.device(q.device):
+        lse = L.reshape(q.shape[0], q.shape[1]).to(torch.float32).contiguous()
+        dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+        dk = torch.empty_strided(k.shape, k.stride(), dtype=k.dtype, device=k.device)
+        dv = torch.empty_strided(k.shape, k.stride(), dtype=k.dtype, device=k.device)
+        ws = torch.empty(q.shape[0] * q.shape[1], dtype=torch.float32, device=q.device)
+        a.o, a.lse, a.dO = o.data_ptr(), lse.data_ptr(), do.data_ptr()
+        a.dq, a.dk, a.dv, a.ws = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr()
+        if L_.fhog_attn_validate(ctypes.byref(a), 1) != 0:
+            return None
+        _lib.check(L_.fhog_attn_bwd(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    return dq, dk, dv
+
+
+def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = False, *, use_hip: Optional[bool] = None):
     """O (dtype of q) and fp32 L = logsumexp_j(scale q.k_j) for (batch, N, d) tensors.
 
     Takes the place of the reference's forward kernel outputs (``fhog/triton_flash.py:123-133``)
     and of ``produce_L`` (``fhog/triton_flash.py:252-258``), with causal support and without an
     (batch, N_Q, N_K) allocation.
+
+    ``use_hip``: None = the HIP kernel when it covers the arguments, else the blocked torch composition;
+    True = the HIP kernel or an error; False = the torch composition.
     """
     if q.dim() == 4:
         B, H = q.shape[:2]
-        o, L = attention_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), scale, causal)
+        o, L = attention_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), scale, causal, use_hip=use_hip)
         return o.view(q.shape), L.view(B, H, -1)
     batch, n_q, d = q.shape
     n_k = k.shape[1]
     if causal and n_q != n_k:
         raise ValueError("causal needs N_Q == N_K")
     scale = d ** -0.5 if scale is None else scale
+    if use_hip is not False:
+        res = _attention_forward_hip(q, k, v, scale, causal)
+        if res is not None:
+            return res
+        if use_hip:
+            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16, d in {64,128}, N multiple of 128, GPU)")
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
@@ -78,10 +155,17 @@ def produce_L(Q, K, is_causal: bool = False):
     return attention_forward(Q, K, K, None, is_causal)[1]
 
 
-def attention_backward(q, k, v, o, do, L, scale: float, causal: bool):
-    """First-order backward (dQ, dK, dV), blocked; the arithmetic of ``fhog/triton_flash.py:201-220``."""
+def attention_backward(q, k, v, o, do, L, scale: float, causal: bool, *, use_hip: Optional[bool] = None):
+    """First-order backward (dQ, dK, dV); the arithmetic of ``fhog/triton_flash.py:201-220`` without the
+    (batch, N_Q, N_K) tensors. ``use_hip`` as in :func:`attention_forward`."""
     batch, n_q, d = q.shape
     n_k = k.shape[1]
+    if use_hip is not False:
+        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal)
+        if res is not None:
+            return res
+        if use_hip:
+            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16, d in {64,128}, N multiple of 128, GPU)")
     dq = torch.empty_like(q)
     dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)

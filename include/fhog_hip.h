@@ -123,6 +123,44 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
    same way: fhog/triton_bwdbwd.py:474-482). */
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream);
 
+/* ---- first-order attention: the callers on either side of the double-backward ---------------------------
+ * bf16 tensors, d in {64, 128}, n_q and n_k multiples of 128 (fhog_attn_supported tells); the layout rules
+ * above apply. O and dO/dQ share the q strides, dK/dV the k strides. */
+typedef struct fhog_attn_args {
+  const void* q;   /* (batch, n_q, d) */
+  const void* k;   /* (batch, n_k, d) */
+  const void* v;   /* (batch, n_k, d) */
+  void* o;         /* (batch, n_q, d): written by fhog_attn_fwd, read by fhog_attn_bwd */
+  float* lse;      /* (batch, n_q) fp32 contiguous: written by fhog_attn_fwd, read by fhog_attn_bwd */
+  const void* dO;  /* backward only */
+  void* dq;        /* backward only, like q */
+  void* dk;        /* backward only, like k */
+  void* dv;        /* backward only, like k */
+  float* ws;       /* backward only: batch * n_q floats */
+  int64_t batch, n_q, n_k, d;
+  int64_t stride_qb, stride_qn, stride_kb, stride_kn;
+  float scale;
+  int32_t dtype;   /* FHOG_DTYPE_BF16 */
+  int32_t causal;  /* as in fhog_bwdbwd_args */
+  int32_t reserved;
+} fhog_attn_args;
+
+size_t fhog_attn_args_size(void);
+
+/* Host-only: FHOG_OK if fhog_attn_fwd / fhog_attn_bwd cover these arguments (backward != 0 also checks the
+   backward-only pointers), else the FHOG_E_* code they would return. */
+int fhog_attn_validate(const fhog_attn_args* args, int backward);
+
+/* O = softmax(scale q k^T [causal]) v and L = logsumexp of the scaled scores over visible keys, one sweep,
+   online soft-max. Replaces flash_kernel (fhog/triton_flash.py:12-133) and, through L, produce_L
+   (fhog/triton_flash.py:252-258). */
+int fhog_attn_fwd(const fhog_attn_args* args, void* hip_stream);
+
+/* dQ, dK, dV of the forward above from (q, k, v, o, dO, lse): the arithmetic of flash_backward_torch
+   (fhog/triton_flash.py:201-220) as three launches (row sums of o*dO, a Q-tiled sweep for dQ, a K-tiled
+   sweep for dK and dV), without the (batch, n_q, n_k) tensors. */
+int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream);
+
 /* Message for the last failing call on this thread ("" if none). */
 const char* fhog_last_error(void);
 

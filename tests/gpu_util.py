@@ -30,7 +30,7 @@ def make_case(batch, n_q, n_k, d, dtype, seed, grad_std=1.0, k_row_scale=False, 
 def with_caches(x, scale, causal):
     """Add O (input dtype) and fp32 L from an fp32 forward on the rounded inputs."""
     import fhog
-    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal)
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, use_hip=False)  # fp32 forward on the rounded inputs
     return dict(x, O=o, L=L)
 
 

@@ -32,15 +32,15 @@ def test_header_symbols_exported(L):
     header = (ROOT / "include" / "fhog_hip.h").read_text()
     names = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(fhog_\w+)\s*\(", header, flags=re.M)
     assert set(names) >= {"fhog_abi_version", "fhog_bwdbwd_args_size", "fhog_bwdbwd_workspace_bytes", "fhog_validate", "fhog_select_impl",
-                          "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error"}
+                          "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error",
+                          "fhog_attn_args_size", "fhog_attn_validate", "fhog_attn_fwd", "fhog_attn_bwd"}
     for n in names:
         assert hasattr(L, n), n
 
 
-def test_struct_mirror_matches_header():
-    from fhog import _lib
+def _header_fields(struct_name):
     header = (ROOT / "include" / "fhog_hip.h").read_text()
-    body = header[header.index("typedef struct fhog_bwdbwd_args"):header.index("} fhog_bwdbwd_args;")]
+    body = header[header.index(f"typedef struct {struct_name}"):header.index(f"}} {struct_name};")]
     body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
     fields = []
     for decl in body.split("{", 1)[1].split(";"):
@@ -49,8 +49,50 @@ def test_struct_mirror_matches_header():
             continue
         for piece in decl.split(","):
             fields.append(re.findall(r"(\w+)\s*$", piece.strip())[0])
-    assert fields == [f[0] for f in _lib.BwdBwdArgs._fields_]
+    return fields
+
+
+def test_struct_mirror_matches_header():
+    from fhog import _lib
+    assert _header_fields("fhog_bwdbwd_args") == [f[0] for f in _lib.BwdBwdArgs._fields_]
     assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 200
+    assert _header_fields("fhog_attn_args") == [f[0] for f in _lib.AttnArgs._fields_]
+    assert ctypes.sizeof(_lib.AttnArgs) == _lib.lib().fhog_attn_args_size() == 160
+
+
+def good_attn_args():
+    from fhog import _lib
+    a = _lib.AttnArgs()
+    for i, (name, _) in enumerate(_lib.AttnArgs._fields_[:10]):
+        setattr(a, name, 0x10000 * (i + 1))
+    a.batch, a.n_q, a.n_k, a.d = 4, 256, 512, 64
+    a.stride_qn = a.stride_kn = 64
+    a.stride_qb, a.stride_kb = 256 * 64, 512 * 64
+    a.scale, a.dtype, a.causal = 0.125, 0, 0
+    return a
+
+
+@pytest.mark.parametrize("mutate, backward, code, word", [
+    (lambda a: None, 1, 0, ""),
+    (lambda a: setattr(a, "dO", 0), 0, 0, ""),            # forward does not look at the backward-only pointers
+    (lambda a: setattr(a, "dO", 0), 1, -1, "dO"),
+    (lambda a: setattr(a, "lse", 0), 0, -1, "lse"),
+    (lambda a: setattr(a, "dtype", 1), 0, -3, "bf16"),
+    (lambda a: setattr(a, "n_q", 200), 0, -2, "multiples of 128"),
+    (lambda a: setattr(a, "d", 32), 0, -2, "d in"),
+    (lambda a: setattr(a, "causal", 1), 0, -6, "causal"),
+    (lambda a: setattr(a, "stride_kn", 60), 0, -4, "stride"),
+    (lambda a: setattr(a, "v", 0x30008), 0, -5, "aligned"),
+    (lambda a: setattr(a, "scale", float("inf")), 0, -9, "scale"),
+])
+def test_attn_validate(L, mutate, backward, code, word):
+    a = good_attn_args()
+    mutate(a)
+    assert L.fhog_attn_validate(ctypes.byref(a), backward) == code
+    if code:
+        assert word in L.fhog_last_error().decode()
+        # the compute entry points refuse the same way, before any launch
+        assert (L.fhog_attn_bwd if backward else L.fhog_attn_fwd)(ctypes.byref(a), None) == code
 
 
 def test_version_and_workspace(L):
