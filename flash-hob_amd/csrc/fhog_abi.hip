@@ -27,7 +27,8 @@ int validate(const fhog_bwdbwd_args* a) {
   const char* names[] = {"q", "k", "v", "o", "dO", "ddq", "ddk", "ddv", "lse", "dq2", "dk2", "dv2", "ddo", "ws"};
   for (int i = 0; i < 14; i++)
     if (!ptrs[i]) return fail(FHOG_E_NULL, "pointer '%s' is NULL", names[i]);
-  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
+  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP32 && a->dtype != FHOG_DTYPE_FP16)
+    return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
   if (a->impl != FHOG_IMPL_AUTO && a->impl != FHOG_IMPL_FP32 && a->impl != FHOG_IMPL_BF16)
     return fail(FHOG_E_DTYPE, "unknown impl %d", a->impl);
   if (a->schedule != FHOG_SCHEDULE_FOUR_PASS && a->schedule != FHOG_SCHEDULE_FUSED_STATS)
@@ -43,7 +44,7 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->causal && a->n_q != a->n_k)
     return fail(FHOG_E_CAUSAL, "causal needs n_q == n_k (got %lld, %lld)", (long long)a->n_q, (long long)a->n_k);
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
-  const int vec = a->dtype == FHOG_DTYPE_BF16 ? 8 : 4;  // elements per 16 bytes
+  const int vec = a->dtype == FHOG_DTYPE_FP32 ? 4 : 8;  // elements per 16 bytes
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
   if (a->stride_qn % vec || a->stride_kn % vec || a->stride_qb % vec || a->stride_kb % vec)
     return fail(FHOG_E_STRIDE, "strides must be multiples of %d elements (16 bytes)", vec);
@@ -52,7 +53,7 @@ int validate(const fhog_bwdbwd_args* a) {
   for (int i = 0; i < 14; i++)
     if (!aligned16(ptrs[i])) return fail(FHOG_E_ALIGN, "pointer '%s' is not 16-byte aligned", names[i]);
   if (a->impl == FHOG_IMPL_BF16) {
-    if (a->dtype != FHOG_DTYPE_BF16) return fail(FHOG_E_DTYPE, "impl=bf16 needs bf16 tensors");
+    if (a->dtype == FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "impl=bf16 needs bf16 or fp16 tensors");
     if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
       return fail(FHOG_E_SHAPE, "impl=bf16 needs d in {64,128} and n_q, n_k multiples of 128");
   }
@@ -62,7 +63,7 @@ int validate(const fhog_bwdbwd_args* a) {
 int select_impl(const fhog_bwdbwd_args* a) {
   if (a->impl == FHOG_IMPL_FP32) return FHOG_IMPL_FP32;
   if (a->impl == FHOG_IMPL_BF16) return FHOG_IMPL_BF16;
-  if (a->dtype == FHOG_DTYPE_BF16 && fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal)) return FHOG_IMPL_BF16;
+  if (a->dtype != FHOG_DTYPE_FP32 && fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal)) return FHOG_IMPL_BF16;
   return FHOG_IMPL_FP32;
 }
 
@@ -95,6 +96,7 @@ fhog::Params to_params(const fhog_bwdbwd_args* a) {
   p.d = (int32_t)a->d;
   p.scale = a->scale;
   p.causal = a->causal;
+  p.f16 = a->dtype == FHOG_DTYPE_FP16;
   return p;
 }
 
@@ -122,7 +124,8 @@ int validate_attn(const fhog_attn_args* a, int backward) {
     if (!ptrs[i]) return fail(FHOG_E_NULL, "pointer '%s' is NULL", names[i]);
     if (!aligned16(ptrs[i])) return fail(FHOG_E_ALIGN, "pointer '%s' is not 16-byte aligned", names[i]);
   }
-  if (a->dtype != FHOG_DTYPE_BF16) return fail(FHOG_E_DTYPE, "the first-order kernels take bf16 tensors (dtype %d given)", a->dtype);
+  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP16)
+    return fail(FHOG_E_DTYPE, "the first-order kernels take bf16 or fp16 tensors (dtype %d given)", a->dtype);
   if (a->batch < 1 || a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld outside 1..65535", (long long)a->batch);
   if (a->n_q < 1 || a->n_k < 1 || a->n_q > (1 << 24) || a->n_k > (1 << 24) || a->batch * a->n_q >= (int64_t)1 << 31)
     return fail(FHOG_E_SHAPE, "n_q/n_k out of range");
@@ -161,6 +164,7 @@ fhog::AttnParams to_attn_params(const fhog_attn_args* a) {
   p.d = (int32_t)a->d;
   p.scale = a->scale;
   p.causal = a->causal;
+  p.f16 = a->dtype == FHOG_DTYPE_FP16;
   return p;
 }
 
@@ -193,7 +197,7 @@ int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream) {
   rd.batch = p.batch;
   rd.n_q = p.n_q;
   rd.d = p.d;
-  hipError_t e = fhog::launch_rowdot(rd, FHOG_DTYPE_BF16, (hipStream_t)hip_stream);
+  hipError_t e = fhog::launch_rowdot(rd, args->dtype, (hipStream_t)hip_stream);
   for (int which = 1; which <= 2 && e == hipSuccess; which++) e = fhog::launch_attn_bf16(p, which, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "attention backward: HIP error %d (%s)", (int)e, hipGetErrorString(e));
   return FHOG_OK;

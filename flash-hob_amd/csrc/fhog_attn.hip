@@ -30,20 +30,16 @@ __device__ __forceinline__ int tr_lane_off_acc(int cb, int s, int lane) {
   return tile_off<D>(r, col >> 3) + ((col >> 2) & 1) * 8;
 }
 
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
-  bf16x2_t v = {(__bf16)lo, (__bf16)hi};
-  return __builtin_bit_cast(uint32_t, v);
-}
 // registers 8t .. 8t+7 of an S-shaped fp32 tile as the bf16 B operand of second-level k-step t
+template <bool F16>
 __device__ __forceinline__ bf16x8_t pack_operand(const f32x16_t& x, int t) {
-  u32x4_t u = {pack2(x[8 * t + 0], x[8 * t + 1]), pack2(x[8 * t + 2], x[8 * t + 3]), pack2(x[8 * t + 4], x[8 * t + 5]),
-               pack2(x[8 * t + 6], x[8 * t + 7])};
+  u32x4_t u = {pack2<F16>(x[8 * t + 0], x[8 * t + 1]), pack2<F16>(x[8 * t + 2], x[8 * t + 3]),
+               pack2<F16>(x[8 * t + 4], x[8 * t + 5]), pack2<F16>(x[8 * t + 6], x[8 * t + 7])};
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
 // acc[cb] += tile^T (columns 32cb..32cb+31) x operand, for both k-steps and all column blocks of the tile
-template <int D, int NOP>
+template <bool F16, int D, int NOP>
 __device__ __forceinline__ void second_level(const char* const (&tile)[NOP], const int (&troff)[D / 32][2],
                                              const bf16x8_t (&op)[NOP][2], f32x16_t (&acc)[NOP][D / 32]) {
   constexpr int NC = D / 32, NIT = 2 * NC;
@@ -61,13 +57,13 @@ __device__ __forceinline__ void second_level(const char* const (&tile)[NOP], con
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int x = 0; x < NOP; x++) acc[x][cb] = mfma(a[c][x], op[x][t], acc[x][cb]);
+    for (int x = 0; x < NOP; x++) acc[x][cb] = mfma<F16>(a[c][x], op[x][t], acc[x][cb]);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
 
 // first-level product of one streamed tile with resident rows: out += tile x res^T (streamed rows = M)
-template <int D, int NRES>
+template <bool F16, int D, int NRES>
 __device__ __forceinline__ void first_level(const char* tile, const int (&aoff)[D / 16], const bf16x8_t* const (&res)[NRES],
                                             f32x16_t (&out)[NRES]) {
   constexpr int KK = D / 16, PF = 2, NB = PF + 1;
@@ -79,13 +75,13 @@ __device__ __forceinline__ void first_level(const char* tile, const int (&aoff)[
     if (kk + PF < KK) a[(kk + PF) % NB] = lds_read128(tile, aoff[kk + PF]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int x = 0; x < NRES; x++) out[x] = mfma(a[kk % NB], res[x][kk], out[x]);
+    for (int x = 0; x < NRES; x++) out[x] = mfma<F16>(a[kk % NB], res[x][kk], out[x]);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
 
 // ---- forward -----------------------------------------------------------------------------------------
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
@@ -138,7 +134,7 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
       const char* stage = smem + (j & 1) * STAGE;
       f32x16_t s[1] = {f32x16_t{0}};
       const bf16x8_t* const res[1] = {Qb};
-      first_level<D, 1>(stage, aoff, res, s);  // S^T: s[r] = (key k0 + 8(r/4) + 4h + r%4, query qi)
+      first_level<F16, D, 1>(stage, aoff, res, s);  // S^T: s[r] = (key k0 + 8(r/4) + 4h + r%4, query qi)
       f32x16_t x;
 #pragma unroll
       for (int r = 0; r < 16; r++) x[r] = s[0][r] * c_scale_log2;
@@ -167,9 +163,9 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
           for (int r = 0; r < 16; r++) acc[0][cb][r] *= alpha;
       }
       m = m_new;
-      const bf16x8_t op[1][2] = {{pack_operand(x, 0), pack_operand(x, 1)}};
+      const bf16x8_t op[1][2] = {{pack_operand<F16>(x, 0), pack_operand<F16>(x, 1)}};
       const char* const vt[1] = {stage + TILE};
-      second_level<D, 1>(vt, troff, op, acc);  // O^T += V^T P^T
+      second_level<F16, D, 1>(vt, troff, op, acc);  // O^T += V^T P^T
     }
     dma_wait();
     __syncthreads();
@@ -181,16 +177,15 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   for (int cb = 0; cb < NC; cb++)
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      bf16x4_t v;
-#pragma unroll
-      for (int e = 0; e < 4; e++) v[e] = (__bf16)(acc[0][cb][4 * g + e] * inv);
-      *reinterpret_cast<bf16x4_t*>(o + 32 * cb + 8 * g + 4 * h) = v;
+      const f32x16_t& a = acc[0][cb];
+      *reinterpret_cast<u32x2_t*>(o + 32 * cb + 8 * g + 4 * h) =
+          pack4<F16>(a[4 * g] * inv, a[4 * g + 1] * inv, a[4 * g + 2] * inv, a[4 * g + 3] * inv);
     }
   if (h == 0) p.lse[(int64_t)bh * p.n_q + qi] = (m + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;  // v_log_f32 is log2
 }
 
 // ---- backward, Q-tiled: dQ -----------------------------------------------------------------------------
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
@@ -246,8 +241,8 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
       f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
       const bf16x8_t* const rq[1] = {Qb};
       const bf16x8_t* const rdo[1] = {dOb};
-      first_level<D, 1>(stage, aoff, rq, s);           // S^T  = K Q^T
-      first_level<D, 1>(stage + TILE, aoff, rdo, dp);  // dP^T = V dO^T
+      first_level<F16, D, 1>(stage, aoff, rq, s);           // S^T  = K Q^T
+      first_level<F16, D, 1>(stage + TILE, aoff, rdo, dp);  // dP^T = V dO^T
       f32x16_t ds;
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * (dp[0][r] - dsum);
@@ -256,9 +251,9 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; r++) ds[r] = (8 * (r / 4) + (r % 4) <= lim) ? ds[r] : 0.f;
       }
-      const bf16x8_t op[1][2] = {{pack_operand(ds, 0), pack_operand(ds, 1)}};
+      const bf16x8_t op[1][2] = {{pack_operand<F16>(ds, 0), pack_operand<F16>(ds, 1)}};
       const char* const kt[1] = {stage};
-      second_level<D, 1>(kt, troff, op, acc);  // dQ^T += K^T dS^T
+      second_level<F16, D, 1>(kt, troff, op, acc);  // dQ^T += K^T dS^T
     }
     dma_wait();
     __syncthreads();
@@ -268,15 +263,14 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
   for (int cb = 0; cb < NC; cb++)
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      bf16x4_t v;
-#pragma unroll
-      for (int e = 0; e < 4; e++) v[e] = (__bf16)(acc[0][cb][4 * g + e] * p.scale);
-      *reinterpret_cast<bf16x4_t*>(o + 32 * cb + 8 * g + 4 * h) = v;
+      const f32x16_t& a = acc[0][cb];
+      *reinterpret_cast<u32x2_t*>(o + 32 * cb + 8 * g + 4 * h) =
+          pack4<F16>(a[4 * g] * p.scale, a[4 * g + 1] * p.scale, a[4 * g + 2] * p.scale, a[4 * g + 3] * p.scale);
     }
 }
 
 // ---- backward, K-tiled: dK, dV ---------------------------------------------------------------------------
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
@@ -352,8 +346,8 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
       f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
       const bf16x8_t* const rk[1] = {Kb};
       const bf16x8_t* const rv[1] = {Vb};
-      first_level<D, 1>(stage, aoff, rk, s);           // S  = Q K^T : s[r] = (query qb + 8(r/4) + 4h + r%4, key kj)
-      first_level<D, 1>(stage + TILE, aoff, rv, dp);   // dP = dO V^T
+      first_level<F16, D, 1>(stage, aoff, rk, s);           // S  = Q K^T : s[r] = (query qb + 8(r/4) + 4h + r%4, key kj)
+      first_level<F16, D, 1>(stage + TILE, aoff, rv, dp);   // dP = dO V^T
       f32x16_t pv, ds;
 #pragma unroll
       for (int g = 0; g < 4; g++) {
@@ -373,9 +367,9 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] *= pv[r];
-      const bf16x8_t op[2][2] = {{pack_operand(ds, 0), pack_operand(ds, 1)}, {pack_operand(pv, 0), pack_operand(pv, 1)}};
+      const bf16x8_t op[2][2] = {{pack_operand<F16>(ds, 0), pack_operand<F16>(ds, 1)}, {pack_operand<F16>(pv, 0), pack_operand<F16>(pv, 1)}};
       const char* const tl[2] = {stage, stage + TILE};
-      second_level<D, 2>(tl, troff, op, acc);  // dK^T += Q^T dS ; dV^T += dO^T P
+      second_level<F16, D, 2>(tl, troff, op, acc);  // dK^T += Q^T dS ; dV^T += dO^T P
     }
     if (j + 1 < t_end) {
       wait_vm0();
@@ -390,14 +384,11 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   for (int cb = 0; cb < NC; cb++)
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      bf16x4_t a, b;
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        a[e] = (__bf16)(acc[0][cb][4 * g + e] * p.scale);
-        b[e] = (__bf16)acc[1][cb][4 * g + e];
-      }
-      *reinterpret_cast<bf16x4_t*>(odk + 32 * cb + 8 * g + 4 * h) = a;
-      *reinterpret_cast<bf16x4_t*>(odv + 32 * cb + 8 * g + 4 * h) = b;
+      const f32x16_t& a = acc[0][cb];
+      const f32x16_t& b = acc[1][cb];
+      *reinterpret_cast<u32x2_t*>(odk + 32 * cb + 8 * g + 4 * h) =
+          pack4<F16>(a[4 * g] * p.scale, a[4 * g + 1] * p.scale, a[4 * g + 2] * p.scale, a[4 * g + 3] * p.scale);
+      *reinterpret_cast<u32x2_t*>(odv + 32 * cb + 8 * g + 4 * h) = pack4<F16>(b[4 * g], b[4 * g + 1], b[4 * g + 2], b[4 * g + 3]);
     }
 }
 
@@ -409,14 +400,13 @@ hipError_t launch(K kernel, unsigned grid, int smem, hipStream_t s, const AttnPa
   return hipGetLastError();
 }
 
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
-  const unsigned heads8 = (unsigned)((p.batch + 7) / 8 * 8);
   constexpr int TILE = TS * 2 * D;
   switch (which) {
-    case 0: return launch(attn_fwd_bf16<D, CAUSAL>, heads8 * (p.n_q / WG_ROWS), 2 * 2 * TILE, s, p);
-    case 1: return launch(attn_bwd_q_bf16<D, CAUSAL>, heads8 * (p.n_q / WG_ROWS), 2 * 2 * TILE, s, p);
-    default: return launch(attn_bwd_k_bf16<D, CAUSAL>, heads8 * (p.n_k / WG_ROWS), 2 * (2 * TILE + 2 * TS * 4), s, p);
+    case 0: return launch(attn_fwd_bf16<F16, D, CAUSAL>, grid_blocks(p.n_q / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    case 1: return launch(attn_bwd_q_bf16<F16, D, CAUSAL>, grid_blocks(p.n_q / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    default: return launch(attn_bwd_k_bf16<F16, D, CAUSAL>, grid_blocks(p.n_k / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
   }
 }
 
@@ -425,8 +415,12 @@ hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
 // which: 0 forward, 1 backward Q-tiled (dQ), 2 backward K-tiled (dK, dV)
 hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
-  if (p.d == 128) return p.causal ? launch_attn_d<128, true>(p, which, s) : launch_attn_d<128, false>(p, which, s);
-  return p.causal ? launch_attn_d<64, true>(p, which, s) : launch_attn_d<64, false>(p, which, s);
+  if (p.f16) {
+    if (p.d == 128) return p.causal ? launch_attn_d<true, 128, true>(p, which, s) : launch_attn_d<true, 128, false>(p, which, s);
+    return p.causal ? launch_attn_d<true, 64, true>(p, which, s) : launch_attn_d<true, 64, false>(p, which, s);
+  }
+  if (p.d == 128) return p.causal ? launch_attn_d<false, 128, true>(p, which, s) : launch_attn_d<false, 128, false>(p, which, s);
+  return p.causal ? launch_attn_d<false, 64, true>(p, which, s) : launch_attn_d<false, 64, false>(p, which, s);
 }
 
 }  // namespace fhog

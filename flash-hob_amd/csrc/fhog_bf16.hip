@@ -22,7 +22,7 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-template <int D, int PASS, bool CAUSAL>
+template <bool F16, int D, int PASS, bool CAUSAL>
 __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
@@ -101,14 +101,14 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
           a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
         __builtin_amdgcn_sched_barrier(0);
         if (ph == 0) {
-          s = mfma(a[c], Qb[kk], s);
-          dds = mfma(a[c], ddQb[kk], dds);
+          s = mfma<F16>(a[c], Qb[kk], s);
+          dds = mfma<F16>(a[c], ddQb[kk], dds);
         } else if (ph == 1) {
-          dp = mfma(a[c], dOb[kk], dp);
+          dp = mfma<F16>(a[c], dOb[kk], dp);
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
         } else if (ph == 2) {
-          dds = mfma(a[c], Qb[kk], dds);
+          dds = mfma<F16>(a[c], Qb[kk], dds);
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 1) {
@@ -119,7 +119,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
             }
           }
         } else {
-          e = mfma(a[c], dOb[kk], e);
+          e = mfma<F16>(a[c], dOb[kk], e);
           if (kk == 0 && CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
             const int lim = qi - k0 - 4 * h;
 #pragma unroll
@@ -172,28 +172,27 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   }
 }
 
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(256);
-  const int heads8 = (p.batch + 7) / 8 * 8;
-  const dim3 grid((unsigned)(heads8 * (p.n_q / WG_ROWS)));
+  const dim3 grid(grid_blocks(p.n_q / WG_ROWS, p.batch));
   const int tile = TS * 2 * D;
   hipError_t e;
   if (pass == FHOG_PASS_DD) {
     const int smem = 2 * 2 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 1, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 1, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<D, 1, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 1, CAUSAL>), grid, block, smem, s, p);
   } else if (pass == FHOG_PASS_B) {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 2, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 2, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<D, 2, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 2, CAUSAL>), grid, block, smem, s, p);
   } else {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<D, 5, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 5, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<D, 5, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 5, CAUSAL>), grid, block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -211,8 +210,12 @@ hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
   if (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV) return launch_bf16_pc_pass(p, pass, s);
   if (pass != FHOG_PASS_DD && pass != FHOG_PASS_B && pass != FHOG_PASS_DD_B) return hipErrorInvalidValue;
-  if (p.d == 128) return p.causal ? launch_stats_d<128, true>(p, pass, s) : launch_stats_d<128, false>(p, pass, s);
-  return p.causal ? launch_stats_d<64, true>(p, pass, s) : launch_stats_d<64, false>(p, pass, s);
+  if (p.f16) {
+    if (p.d == 128) return p.causal ? launch_stats_d<true, 128, true>(p, pass, s) : launch_stats_d<true, 128, false>(p, pass, s);
+    return p.causal ? launch_stats_d<true, 64, true>(p, pass, s) : launch_stats_d<true, 64, false>(p, pass, s);
+  }
+  if (p.d == 128) return p.causal ? launch_stats_d<false, 128, true>(p, pass, s) : launch_stats_d<false, 128, false>(p, pass, s);
+  return p.causal ? launch_stats_d<false, 64, true>(p, pass, s) : launch_stats_d<false, 64, false>(p, pass, s);
 }
 
 }  // namespace fhog

@@ -44,12 +44,7 @@ struct PCSmem {
 //   steps 24..31  A = ddV: E += ddV dO^T         + ddP = P (ddS - dd), z = P (ddS u - v)
 //   tail                                          dS' = P E + z     [= P (E + dP (ddS - dd) - ddS d - b)]
 // LDS operands are fetched PF steps ahead. Results go to the operand tiles dS, dS', ddP, P.
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  bf16x2_t v = {(__bf16)a, (__bf16)b};
-  return __builtin_bit_cast(uint32_t, v);
-}
 // registers 4g..4g+3 of one S-shaped tile, given as packed pairs pk[2g], pk[2g+1]
 __device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int lane) {
   const int n = lane & 31, h = lane >> 5;
@@ -60,7 +55,7 @@ __device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int
   }
 }
 
-template <int D>
+template <bool F16, int D>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
                                           const bf16x8_t* dOb, int lane, int q_idx, int k_base, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
@@ -86,14 +81,14 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
     if (i + PF < NSTEP) a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
     __builtin_amdgcn_sched_barrier(0);
     if (ph == 0) {
-      s = mfma(a[c], Qb[kk], s);
-      dds = mfma(a[c], ddQb[kk], dds);
+      s = mfma<F16>(a[c], Qb[kk], s);
+      dds = mfma<F16>(a[c], ddQb[kk], dds);
     } else if (ph == 1) {
-      dp = mfma(a[c], dOb[kk], dp);
+      dp = mfma<F16>(a[c], dOb[kk], dp);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
     } else if (ph == 2) {
-      dds = mfma(a[c], Qb[kk], dds);
+      dds = mfma<F16>(a[c], Qb[kk], dds);
       if (kk == 0 && mask) {  // wave-uniform: only the block on the diagonal
         const int lim = q_idx - k_base - 4 * h;
 #pragma unroll
@@ -102,18 +97,18 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
         const float u0 = dp[r] - dsum, u1 = dp[r + 1] - dsum;
-        pk_ds[r / 2] = pack2(pv[r] * u0, pv[r + 1] * u1);
+        pk_ds[r / 2] = pack2<F16>(pv[r] * u0, pv[r + 1] * u1);
         vv[r] = __builtin_fmaf(dp[r], dd, b);
         vv[r + 1] = __builtin_fmaf(dp[r + 1], dd, b);
         us[r] = u0 * scale;
         us[r + 1] = u1 * scale;
       }
     } else {
-      e = mfma(a[c], dOb[kk], e);
+      e = mfma<F16>(a[c], dOb[kk], e);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
-        pk_ddp[r / 2] = pack2(pv[r] * __builtin_fmaf(dds[r], scale, -dd), pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd));
-        pk_p[r / 2] = pack2(pv[r], pv[r + 1]);
+        pk_ddp[r / 2] = pack2<F16>(pv[r] * __builtin_fmaf(dds[r], scale, -dd), pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd));
+        pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
         vv[r] = pv[r] * __builtin_fmaf(dds[r], us[r], -vv[r]);              // z
         vv[r + 1] = pv[r + 1] * __builtin_fmaf(dds[r + 1], us[r + 1], -vv[r + 1]);
       }
@@ -125,12 +120,12 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
   sop_write_pk(sop + 3 * SOP_TILE, pk_p, lane);
 #pragma unroll
   for (int r = 0; r < 16; r += 2)
-    pk_ds2[r / 2] = pack2(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
+    pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
   sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, lane);
 }
 
 
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   using SM = PCSmem<D, false>;
@@ -164,7 +159,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       if (j < n_tiles && (!CAUSAL || k0 <= qw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        produce_q<D>(stage, sop, Qb, ddQb, dOb, lane, qi, k0, CAUSAL && k0 == qw, c_scale_log2, l_log2, p.scale, dsum, dd, b);
+        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, qi, k0, CAUSAL && k0 == qw, c_scale_log2, l_log2, p.scale, dsum, dd, b);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -244,17 +239,17 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
             }
             __builtin_amdgcn_sched_barrier(0);
             if (act0) {
-              acc_dq[0][cl] = mfma(a_op[0][0], bop[c][1], acc_dq[0][cl]);
-              acc_ddo[0][cl] = mfma(a_op[0][2], bop[c][2], acc_ddo[0][cl]);
+              acc_dq[0][cl] = mfma<F16>(a_op[0][0], bop[c][1], acc_dq[0][cl]);
+              acc_ddo[0][cl] = mfma<F16>(a_op[0][2], bop[c][2], acc_ddo[0][cl]);
             }
-            acc_dq[1][cl] = mfma(a_op[1][0], bop[c][1], acc_dq[1][cl]);
-            acc_ddo[1][cl] = mfma(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
+            acc_dq[1][cl] = mfma<F16>(a_op[1][0], bop[c][1], acc_dq[1][cl]);
+            acc_ddo[1][cl] = mfma<F16>(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
             if (act0) {
-              acc_dq[0][cl] = mfma(a_op[0][1], bop[c][0], acc_dq[0][cl]);
-              acc_ddo[0][cl] = mfma(a_op[0][3], bop[c][3], acc_ddo[0][cl]);
+              acc_dq[0][cl] = mfma<F16>(a_op[0][1], bop[c][0], acc_dq[0][cl]);
+              acc_ddo[0][cl] = mfma<F16>(a_op[0][3], bop[c][3], acc_ddo[0][cl]);
             }
-            acc_dq[1][cl] = mfma(a_op[1][1], bop[c][0], acc_dq[1][cl]);
-            acc_ddo[1][cl] = mfma(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
+            acc_dq[1][cl] = mfma<F16>(a_op[1][1], bop[c][0], acc_dq[1][cl]);
+            acc_ddo[1][cl] = mfma<F16>(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
@@ -265,8 +260,8 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
     // acc[qb][cl][r] holds (query qw0 + 32 qb + 8*(r/4) + 4h + r%4, column 32*(NCL*ch + cl) + n)
-    __bf16* odq = (__bf16*)p.dq2 + qoff;
-    __bf16* oddo = (__bf16*)p.ddo + qoff;
+    uint16_t* odq = (uint16_t*)p.dq2 + qoff;
+    uint16_t* oddo = (uint16_t*)p.ddo + qoff;
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
@@ -274,14 +269,14 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int64_t o = (int64_t)(qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_qn + 32 * (NCL * ch + cl) + n;
-          odq[o] = (__bf16)(acc_dq[qb][cl][r] * p.scale);
-          oddo[o] = (__bf16)acc_ddo[qb][cl][r];
+          odq[o] = to_elem<F16>(acc_dq[qb][cl][r] * p.scale);
+          oddo[o] = to_elem<F16>(acc_ddo[qb][cl][r]);
         }
   }
 }
 
 // ---- pass 4 ------------------------------------------------------------------------------------------
-template <int D>
+template <bool F16, int D>
 __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* ddKb,
                                           const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int k_idx, int q_base,
                                           bool mask, float c_scale_log2, float scale) {
@@ -309,11 +304,11 @@ __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf
       a[c ^ 1][2] = lds_read128(tdO, off);
     }
     __builtin_amdgcn_sched_barrier(0);
-    s = mfma(a[c][0], Kb[kk], s);
-    dds = mfma(a[c][1], Kb[kk], dds);
-    dp = mfma(a[c][2], Vb[kk], dp);
-    dds = mfma(a[c][0], ddKb[kk], dds);
-    e = mfma(a[c][2], ddVb[kk], e);
+    s = mfma<F16>(a[c][0], Kb[kk], s);
+    dds = mfma<F16>(a[c][1], Kb[kk], dds);
+    dp = mfma<F16>(a[c][2], Vb[kk], dp);
+    dds = mfma<F16>(a[c][0], ddKb[kk], dds);
+    e = mfma<F16>(a[c][2], ddVb[kk], e);
     __builtin_amdgcn_sched_barrier(0);
   }
   f32x16_t pv, dsv, ds2v, ddpv;
@@ -345,12 +340,12 @@ __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf
       ds2v[r] = p * (dp2 - b4[j]);
     }
   }
-  sop_write(sop + 0 * SOP_TILE, dsv, lane);
-  sop_write(sop + 1 * SOP_TILE, ds2v, lane);
-  sop_write(sop + 2 * SOP_TILE, ddpv, lane);
+  sop_write<F16>(sop + 0 * SOP_TILE, dsv, lane);
+  sop_write<F16>(sop + 1 * SOP_TILE, ds2v, lane);
+  sop_write<F16>(sop + 2 * SOP_TILE, ddpv, lane);
 }
 
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   using SM = PCSmem<D, true>;
@@ -384,7 +379,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       if (j < t_end && (!CAUSAL || qb >= kw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        produce_k<D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, kj, qb, CAUSAL && qb == kw, c_scale_log2, p.scale);
+        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, kj, qb, CAUSAL && qb == kw, c_scale_log2, p.scale);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -466,9 +461,9 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
             bop[c ^ 1][2] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
           }
           __builtin_amdgcn_sched_barrier(0);
-          acc_dk[cb] = mfma(a_op[t][0], bop[c][0], acc_dk[cb]);
-          acc_dv[cb] = mfma(a_op[t][2], bop[c][2], acc_dv[cb]);
-          acc_dk[cb] = mfma(a_op[t][1], bop[c][1], acc_dk[cb]);
+          acc_dk[cb] = mfma<F16>(a_op[t][0], bop[c][0], acc_dk[cb]);
+          acc_dv[cb] = mfma<F16>(a_op[t][2], bop[c][2], acc_dv[cb]);
+          acc_dk[cb] = mfma<F16>(a_op[t][1], bop[c][1], acc_dk[cb]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -478,34 +473,33 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       sc = (sc == RING - 1) ? 0 : sc + 1;
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
-    __bf16* odk = (__bf16*)p.dk2 + koff;
-    __bf16* odv = (__bf16*)p.dv2 + koff;
+    uint16_t* odk = (uint16_t*)p.dk2 + koff;
+    uint16_t* odv = (uint16_t*)p.dv2 + koff;
 #pragma unroll
     for (int cb = 0; cb < NC; cb++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int64_t o = (int64_t)(kw + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_kn + cb * 32 + n;
-        odk[o] = (__bf16)(acc_dk[cb][r] * p.scale);
-        odv[o] = (__bf16)acc_dv[cb][r];
+        odk[o] = to_elem<F16>(acc_dk[cb][r] * p.scale);
+        odv[o] = to_elem<F16>(acc_dv[cb][r]);
       }
   }
 }
 
-template <int D, bool CAUSAL>
+template <bool F16, int D, bool CAUSAL>
 hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(PC_THREADS);
-  const int heads8 = (p.batch + 7) / 8 * 8;
   hipError_t e;
   if (pass == FHOG_PASS_DQ_DDO) {
     const int smem = PCSmem<D, false>::TOTAL;
-    e = hipFuncSetAttribute((const void*)q_sweep3_pc<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep3_pc<D, CAUSAL>), dim3((unsigned)(heads8 * (p.n_q / WG_ROWS))), block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep3_pc<F16, D, CAUSAL>), dim3(grid_blocks(p.n_q / WG_ROWS, p.batch)), block, smem, s, p);
   } else {
     const int smem = PCSmem<D, true>::TOTAL;
-    e = hipFuncSetAttribute((const void*)k_sweep_pc<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_sweep_pc<D, CAUSAL>), dim3((unsigned)(heads8 * (p.n_k / WG_ROWS))), block, smem, s, p);
+    hipLaunchKernelGGL((k_sweep_pc<F16, D, CAUSAL>), dim3(grid_blocks(p.n_k / WG_ROWS, p.batch)), block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -513,8 +507,12 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
 }  // namespace
 
 hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s) {
-  if (p.d == 128) return p.causal ? launch_pc_d<128, true>(p, pass, s) : launch_pc_d<128, false>(p, pass, s);
-  return p.causal ? launch_pc_d<64, true>(p, pass, s) : launch_pc_d<64, false>(p, pass, s);
+  if (p.f16) {
+    if (p.d == 128) return p.causal ? launch_pc_d<true, 128, true>(p, pass, s) : launch_pc_d<true, 128, false>(p, pass, s);
+    return p.causal ? launch_pc_d<true, 64, true>(p, pass, s) : launch_pc_d<true, 64, false>(p, pass, s);
+  }
+  if (p.d == 128) return p.causal ? launch_pc_d<false, 128, true>(p, pass, s) : launch_pc_d<false, 128, false>(p, pass, s);
+  return p.causal ? launch_pc_d<false, 64, true>(p, pass, s) : launch_pc_d<false, 64, false>(p, pass, s);
 }
 
 }  // namespace fhog

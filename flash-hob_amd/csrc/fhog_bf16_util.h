@@ -48,19 +48,40 @@ __device__ __forceinline__ bf16x8_t lds_read_tr_pre(const char* p0, const char* 
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// ---- fp32 -> 16-bit tensor type (bf16, or fp16 when F16), round to nearest even ---------------------------
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (F16) {
+    typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+    f16x2_t v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  } else {
+    typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+    bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+}
+template <bool F16>
+__device__ __forceinline__ u32x2_t pack4(float a, float b, float c, float d) {
+  return u32x2_t{pack2<F16>(a, b), pack2<F16>(c, d)};
+}
+template <bool F16>
+__device__ __forceinline__ uint16_t to_elem(float x) {
+  if constexpr (F16) return __builtin_bit_cast(uint16_t, (_Float16)x);
+  else return __builtin_bit_cast(uint16_t, (__bf16)x);
+}
+
 // ---- S-shaped bf16 operand tiles handed from producer to consumer waves through LDS ------------
 // 32 stationary rows x 32 streamed rows, 64 bytes per row, 16-byte chunks XOR-swizzled by (row>>2)&3.
 constexpr int SOP_TILE = 32 * 64;
 // producer: registers 4g..4g+3 of an S-shaped fp32 tile (streamed rows 8g + 4h + 0..3) of stationary row n
+template <bool F16>
 __device__ __forceinline__ void sop_write(char* tile, const f32x16_t& x, int lane) {
   const int n = lane & 31, h = lane >> 5;
 #pragma unroll
-  for (int g = 0; g < 4; g++) {
-    bf16x4_t v;
-#pragma unroll
-    for (int e = 0; e < 4; e++) v[e] = (__bf16)x[4 * g + e];
-    *reinterpret_cast<bf16x4_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = v;
-  }
+  for (int g = 0; g < 4; g++)
+    *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) =
+        pack4<F16>(x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]);
 }
 // consumer: A operand of second-level step t: stationary row n, streamed rows 16t + 8h + 0..7
 __device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) {
@@ -68,8 +89,15 @@ __device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) 
   return *reinterpret_cast<const bf16x8_t*>(tile + n * 64 + (((2 * t + h) ^ ((n >> 2) & 3)) << 4));
 }
 
+// The kernels carry 16-bit operands as bf16x8_t whatever the tensor type; F16 selects the instruction.
+template <bool F16>
 __device__ __forceinline__ f32x16_t mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  if constexpr (F16) {
+    typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
 }
 
 // ---- direct global -> LDS staging (no registers): global_load_lds_dwordx4 ------------------------
@@ -120,18 +148,29 @@ __device__ __forceinline__ void load_resident(bf16x8_t* dst, const __bf16* base,
   for (int kk = 0; kk < D / 16; kk++) dst[kk] = *reinterpret_cast<const bf16x8_t*>(p + 16 * kk);
 }
 
-// XCD-aware decode of a 1-D grid: workgroup ids go round-robin over the 8 XCDs, so all tiles of
-// one (batch*head) slice are given ids with the same id % 8 and share that XCD's L2.
-// Returns false when the id falls beyond the last slice.
+// XCD-aware 1-D grid. Workgroup ids go round-robin over the 8 XCDs (id % 8 = XCD), each with its own L2.
+// With 8 or more (batch*head) slices every slice is pinned to one XCD, so that all its tiles stream the slice's
+// other side through ONE L2. With fewer slices a slice is spread over 8/batch (rounded down to a power of two)
+// XCDs, tiles interleaved, so that a single long head still fills the chip.
+//   xcds_per_slice XS = 8, 4, 2, 2, 1, ... for batch = 1, 2, 3, 4, >= 5;  slices per round = 8 / XS
+__host__ __device__ __forceinline__ int xcds_per_slice(int batch) { return batch >= 5 ? 1 : batch >= 3 ? 2 : batch == 2 ? 4 : 8; }
+// number of workgroups to launch for n_tiles tiles per slice
+__host__ __forceinline__ unsigned grid_blocks(int n_tiles, int batch) {
+  const int xs = xcds_per_slice(batch), per_round = 8 / xs;
+  const int rounds = (batch + per_round - 1) / per_round, tiles_per_xcd = (n_tiles + xs - 1) / xs;
+  return (unsigned)(rounds * 8 * tiles_per_xcd);
+}
+// Returns false when the id falls beyond the last slice or tile.
 __device__ __forceinline__ bool decode_block(int n_tiles, int batch, bool heavy_first, int& bh, int& tile) {
   const int id = blockIdx.x;
   const int xcd = id & 7, slot = id >> 3;
-  bh = xcd + 8 * (slot / n_tiles);
-  tile = slot % n_tiles;
+  const int xs = xcds_per_slice(batch), per_round = 8 / xs, tiles_per_xcd = (n_tiles + xs - 1) / xs;
+  bh = xcd / xs + per_round * (slot / tiles_per_xcd);
+  tile = (slot % tiles_per_xcd) * xs + xcd % xs;
+  if (bh >= batch || tile >= n_tiles) return false;
   if (heavy_first) tile = n_tiles - 1 - tile;
-  return bh < batch;
+  return true;
 }
-
 
 }  // namespace bf16k
 }  // namespace fhog

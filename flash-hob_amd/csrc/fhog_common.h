@@ -39,6 +39,7 @@ struct Params {
   int32_t batch, n_q, n_k, d;
   float scale;
   int32_t causal;
+  int32_t f16;  // 16-bit tensors are fp16 (else bf16); read by the 16-bit MFMA family only
 };
 
 // Kernel-side view of fhog_attn_args (first-order forward and backward).
@@ -57,6 +58,7 @@ struct AttnParams {
   int32_t batch, n_q, n_k, d;
   float scale;
   int32_t causal;
+  int32_t f16;  // tensors are fp16 (else bf16)
 };
 
 // Launchers implemented in the kernel translation units. Each returns hipGetLastError().

@@ -28,6 +28,13 @@ __device__ inline f32x4_t load4<__bf16>(const __bf16* p) {
   f32x4_t r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
   return r;
 }
+template <>
+__device__ inline f32x4_t load4<_Float16>(const _Float16* p) {
+  typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4_t;
+  f16x4_t v = *reinterpret_cast<const f16x4_t*>(p);
+  f32x4_t r = {(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+  return r;
+}
 template <typename T>
 __device__ inline void store1(T* p, float x) {
   *p = (T)x;
@@ -392,11 +399,13 @@ hipError_t launch_rowdot_t(const Params& p, hipStream_t s) {
 }  // namespace
 
 hipError_t launch_rowdot(const Params& p, int dtype, hipStream_t s) {
-  return dtype == FHOG_DTYPE_FP32 ? launch_rowdot_t<float>(p, s) : launch_rowdot_t<__bf16>(p, s);
+  if (dtype == FHOG_DTYPE_FP32) return launch_rowdot_t<float>(p, s);
+  return dtype == FHOG_DTYPE_FP16 ? launch_rowdot_t<_Float16>(p, s) : launch_rowdot_t<__bf16>(p, s);
 }
 
 hipError_t launch_fp32_pass(const Params& p, int dtype, int pass, hipStream_t s) {
-  return dtype == FHOG_DTYPE_FP32 ? launch_pass_t<float>(p, pass, s) : launch_pass_t<__bf16>(p, pass, s);
+  if (dtype == FHOG_DTYPE_FP32) return launch_pass_t<float>(p, pass, s);
+  return dtype == FHOG_DTYPE_FP16 ? launch_pass_t<_Float16>(p, pass, s) : launch_pass_t<__bf16>(p, pass, s);
 }
 
 }  // namespace fhog

@@ -12,7 +12,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libfhog_hip.so"
 
-DTYPE_BF16, DTYPE_FP32 = 0, 1
+DTYPE_BF16, DTYPE_FP32, DTYPE_FP16 = 0, 1, 2
 IMPL_AUTO, IMPL_FP32, IMPL_BF16 = 0, 1, 2
 PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B = 0, 1, 2, 3, 4, 5
 ABI_VERSION = 1

@@ -10,7 +10,7 @@ commented stub (``fhog/triton_bwdbwd.py:538-554``).  Here it is wired:
     AttnBwd.forward          -> dQ, dK, dV   (first-order backward)
     AttnBwd.backward         -> flash_bwdbwd(...) -> dQ', dK', dV', ddO
 
-The forward and the first-order backward are the callers on either side of the hot path.  For bf16
+The forward and the first-order backward are the callers on either side of the hot path.  For bf16 and fp16
 tensors with d in {64, 128} and sequence lengths that are multiples of 128 they run as HIP kernels of
 the same library (``fhog_attn_fwd`` / ``fhog_attn_bwd``); every other dtype or shape takes
 linear-memory torch compositions on the GPU (blocked over heads and query rows, fp32 accumulation).
@@ -28,6 +28,7 @@ import torch
 from . import _lib
 from .bwdbwd import flash_bwdbwd
 
+_HIP_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
 _BLOCK_ELEMS = 1 << 26  # fp32 elements of one materialised (heads, rows, N_K) block (256 MiB)
 
 
@@ -52,7 +53,7 @@ def _scores(q, k, scale, causal, r0):
 
 def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
     """Arguments for the HIP first-order kernels, or None when they do not cover these tensors."""
-    if not (q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == v.dtype == torch.bfloat16):
+    if not (q.is_cuda and q.dtype in _HIP_DTYPES and k.dtype == v.dtype == q.dtype):
         return None
     a = _lib.AttnArgs()
     a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
@@ -60,7 +61,7 @@ def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
     a.n_k = k.shape[1]
     a.stride_qb, a.stride_qn = q.stride(0), q.stride(1)
     a.stride_kb, a.stride_kn = k.stride(0), k.stride(1)
-    a.scale, a.dtype, a.causal = float(scale), _lib.DTYPE_BF16, int(bool(causal))
+    a.scale, a.dtype, a.causal = float(scale), _HIP_DTYPES[q.dtype], int(bool(causal))
     return a
 
 
@@ -96,7 +97,7 @@ def _attention_backward_hip(q, k, v, o, do, L, scale, causal):
         ts_k = [t.contiguous() for t in ts_k]
     (q, o, do), (k, v) = ts_q, ts_k
     a = _hip_args(q, k, v, scale, causal)
-    if a is None or o.dtype != torch.bfloat16 or do.dtype != torch.bfloat16:
+    if a is None or o.dtype != q.dtype or do.dtype != q.dtype:
         return None
     L_ = _lib.lib()
     with torch.cuda.device(q.device):
@@ -137,7 +138,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = Fal
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16, d in {64,128}, N multiple of 128, GPU)")
+            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16/fp16, d in {64,128}, N multiple of 128, GPU)")
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
@@ -165,7 +166,7 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal: bool, *, use_hip
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16, d in {64,128}, N multiple of 128, GPU)")
+            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16/fp16, d in {64,128}, N multiple of 128, GPU)")
     dq = torch.empty_like(q)
     dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)

@@ -10,7 +10,7 @@ import torch
 
 from . import _lib
 
-_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32}
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32, torch.float16: _lib.DTYPE_FP16}
 _IMPLS = {None: _lib.IMPL_AUTO, "auto": _lib.IMPL_AUTO, "fp32": _lib.IMPL_FP32, "bf16": _lib.IMPL_BF16}
 
 
@@ -74,15 +74,16 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
 
     Args:
         Q, O, dO, ddQ: (batch, N_Q, d) or (B, H, N_Q, d); K, V, ddK, ddV: (batch, N_K, d) or (B, H, N_K, d).
-            bf16 or fp32 (all the same dtype), on a ROCm device.
+            bf16, fp16 or fp32 (all the same dtype), on a ROCm device.
         L: (batch, N_Q) / (B, H, N_Q) log-sum-exp of ``scale * Q K^T`` over visible keys. Used in fp32
             (any other dtype is up-cast; the reference passes it in the input dtype,
             ``fhog/triton_flash.py:255-257``).
         scale: python float.
         causal: keyword only; top-left mask, needs N_Q == N_K. (The reference has no causal
             double-backward.)
-        impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the bf16 MFMA kernels for
-            bf16 tensors whose shape they support, the fp32-MFMA kernels otherwise.
+        impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the 16-bit MFMA kernels ("bf16": products
+            in the tensor type, bf16 or fp16) for 16-bit tensors whose shape they support, the fp32-MFMA kernels
+            otherwise.
         fused_stats: opt-in schedule that takes ``dd`` and ``b`` from one sweep instead of the reference's two
             (``fhog/triton_bwdbwd.py:185-251``): 22 instead of 25 recomputed products; ``b`` then differs from the
             default schedule's value only by fp32 summation order.
@@ -99,7 +100,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
     if not isinstance(L, torch.Tensor):
         raise TypeError(f"L must be a torch.Tensor, got {type(L).__name__}")
     if Q.dtype not in _DTYPES:
-        raise TypeError(f"unsupported dtype {Q.dtype}; expected torch.bfloat16 or torch.float32")
+        raise TypeError(f"unsupported dtype {Q.dtype}; expected torch.bfloat16, torch.float16 or torch.float32")
     for n, t in tensors.items():
         if t.dtype != Q.dtype:
             raise TypeError(f"{n} has dtype {t.dtype}, expected {Q.dtype} like Q")

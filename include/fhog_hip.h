@@ -33,6 +33,7 @@ extern "C" {
 /* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
 #define FHOG_DTYPE_BF16 0
 #define FHOG_DTYPE_FP32 1
+#define FHOG_DTYPE_FP16 2 /* the dtype of the reference's benchmark sweep (fhog/benchhhh.py:15-110) */
 
 /* error codes */
 #define FHOG_OK 0
@@ -56,9 +57,10 @@ extern "C" {
                               (same quantities as fhog/triton_bwdbwd.py:185-251, three recomputed products fewer) */
 
 /* kernel families (fhog_bwdbwd_args.impl) */
-#define FHOG_IMPL_AUTO 0   /* bf16 MFMA kernels when the shape allows, else the fp32-MFMA kernels */
+#define FHOG_IMPL_AUTO 0   /* 16-bit MFMA kernels for bf16/fp16 tensors when the shape allows, else the fp32-MFMA kernels */
 #define FHOG_IMPL_FP32 1   /* force the fp32-MFMA kernels (any dtype; every intermediate in fp32) */
-#define FHOG_IMPL_BF16 2   /* force the bf16 MFMA kernels; error if the shape/dtype does not fit */
+#define FHOG_IMPL_BF16 2   /* force the 16-bit MFMA kernels (bf16 or fp16 tensors, products in the tensor type);
+                              error if the shape/dtype does not fit */
 
 /* pass schedules of fhog_bwdbwd (fhog_bwdbwd_args.schedule) */
 #define FHOG_SCHEDULE_FOUR_PASS 0   /* the reference's schedule: d, then dd, b, dQ2+ddO, dK2+dV2 as four sweeps
@@ -124,7 +126,7 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream);
 
 /* ---- first-order attention: the callers on either side of the double-backward ---------------------------
- * bf16 tensors, d in {64, 128}, n_q and n_k multiples of 128 (fhog_attn_supported tells); the layout rules
+ * bf16 or fp16 tensors, d in {64, 128}, n_q and n_k multiples of 128 (fhog_attn_supported tells); the layout rules
  * above apply. O and dO/dQ share the q strides, dK/dV the k strides. */
 typedef struct fhog_attn_args {
   const void* q;   /* (batch, n_q, d) */
@@ -140,7 +142,7 @@ typedef struct fhog_attn_args {
   int64_t batch, n_q, n_k, d;
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   float scale;
-  int32_t dtype;   /* FHOG_DTYPE_BF16 */
+  int32_t dtype;   /* FHOG_DTYPE_BF16 | FHOG_DTYPE_FP16 */
   int32_t causal;  /* as in fhog_bwdbwd_args */
   int32_t reserved;
 } fhog_attn_args;

@@ -160,7 +160,8 @@ def test_python_wrapper_errors():
     with pytest.raises(TypeError):
         fhog.flash_bwdbwd(q, k, k, q, q, q, k, k.float(), L, 0.125)
     with pytest.raises(TypeError):
-        fhog.flash_bwdbwd(q.half(), k.half(), k.half(), q.half(), q.half(), q.half(), k.half(), k.half(), L, 0.125)
+        d64 = lambda x: x.double()   # fp64 tensors are not taken (bf16, fp16, fp32 are)
+        fhog.flash_bwdbwd(d64(q), d64(k), d64(k), d64(q), d64(q), d64(q), d64(k), d64(k), L, 0.125)
     with pytest.raises(ValueError):
         fhog.flash_bwdbwd(q, k, k, q, q, q, k, t(2, 64, 64), L, 0.125)
     with pytest.raises(ValueError):

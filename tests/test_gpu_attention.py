@@ -62,6 +62,24 @@ def test_backward_against_fp64_oracle(shape, causal):
         assert normalised_max_error(got, want) < 2e-2, name
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp16_forward_and_backward(causal):
+    import fhog
+    from fhog.attention import attention_backward
+    x = make_case(3, 256, 256, 128, torch.float16, seed=27)
+    scale = 128 ** -0.5
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, use_hip=True)
+    o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), scale, causal)
+    assert o.dtype == torch.float16
+    assert normalised_max_error(o, o_ref) < 2e-3
+    assert (L.double().cpu() - torch.from_numpy(l_ref)).abs().max() < 2e-3
+    got = attention_backward(x["Q"], x["K"], x["V"], o, x["dO"], L, scale, causal, use_hip=True)
+    ref = first_backward(_np(x["Q"]), _np(x["K"]), _np(x["V"]), _np(x["dO"]), scale, causal)
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        assert a.dtype == torch.float16
+        assert normalised_max_error(a, b) < 5e-3, name
+
+
 def test_strided_rows_and_4d_input():
     """Row stride larger than d (q, k, v as slices of one packed (batch, N, 3d) tensor) and (B, H, N, d) input."""
     import fhog

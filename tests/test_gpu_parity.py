@@ -167,6 +167,36 @@ def test_bf16_fused_statistics_match_separate_passes(d, causal):
     assert normalised_max_error(fused[2], separate[2]) < 1e-3      # dd_i * sum_j P dP taken out of the sum
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("impl", ["bf16", "fp32"])
+@pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
+def test_fp16_tensors_both_families(shape, impl, causal):
+    """fp16 tensors (the dtype of the reference's benchmark sweep, fhog/benchhhh.py:15-26) through the 16-bit MFMA
+    kernels (products in fp16) and through the fp32-MFMA kernels."""
+    batch, n_q, n_k, d = shape
+    if causal:
+        n_k = n_q
+    x = make_case(batch, n_q, n_k, d, torch.float16, seed=13, grad_std=0.1)
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal)
+    outs = run_fhog(x, scale, causal, impl=impl, return_stats=True)
+    ref = reference_fp64_cpu(x, scale, causal)
+    e = errors(outs[:4], [ref[n] for n in NAMES])
+    assert all(o.dtype == torch.float16 for o in outs[:4])
+    assert max(e.values()) < (5e-3 if impl == "bf16" else 1e-3), e   # fp16 carries 3 more mantissa bits than bf16
+    for got, name in zip(outs[4], ("d", "dd", "b")):
+        assert normalised_max_error(got, ref[name]) < 2e-3, name
+
+
+def test_single_head_spreads_over_the_chip():
+    """batch = 1 (the reference's sweep shape): tiles of the one slice are dealt to all XCDs; results unchanged."""
+    x = with_caches(make_case(1, 1024, 1024, 64, torch.bfloat16, seed=14, grad_std=0.1), 0.125, True)
+    outs = run_fhog(x, 0.125, True, impl="bf16")
+    ref = reference_fp64_cpu(x, 0.125, True)
+    e = errors(outs, [ref[n] for n in NAMES])
+    assert max(e.values()) < 2e-2, e
+
+
 def test_bf16_auto_dispatch():
     from fhog import BwdBwdPlan
     x = with_caches(make_case(2, 256, 256, 64, torch.bfloat16, seed=6), 0.125, False)
