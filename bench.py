@@ -43,6 +43,26 @@ def event_time_ms(fn, iters):
     return e0.elapsed_time(e1) / iters
 
 
+def mfma_sustained(dev):
+    """bf16 MFMA rate of a loop of nothing but MFMAs, on zero and on random operands (TFLOP/s): the rate the chip holds
+    under its power limit depends on the operand data; the second figure is the practical ceiling for real tensors."""
+    import ctypes
+    import torch
+    from fhog import _lib
+    L = _lib.lib()
+    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {}
+    for name, mode in (("zeros", 0), ("random", 1)):
+        flops = ctypes.c_double()
+        run = lambda trips: _lib.check(L.fhog_probe_mfma_rate(out.data_ptr(), blocks, trips, mode, ctypes.byref(flops), stream))
+        run(4000)   # warm-up, also lets the clock settle
+        ms = event_time_ms(lambda: run(20000), 2)
+        res[name] = round(flops.value / ms / 1e9, 1)
+    return res
+
+
 def cpu_baseline(w, x_cpu, heads, repeats):
     """torch autograd double-backward (fp32, materialised, one head at a time) on the host cores."""
     import torch
@@ -152,6 +172,8 @@ def main():
                      "flops_per_launch": dom_flops, "ms_per_launch": round(per_pass[dom], 4),
                      "traffic": TRAFFIC_BYTES.get((w.name, dom))},
     }
+    out["mfma_sustained_tflops"] = mfma_sustained(dev)
+    out["roofline"]["frac_of_sustained_random"] = round(dom_tflops / out["mfma_sustained_tflops"]["random"], 4)
     if args.cpu_heads > 0:
         out["cpu_baseline"] = cpu_baseline(w, x_cpu, min(args.cpu_heads, w.batch), repeats=2)
     print(json.dumps(out))

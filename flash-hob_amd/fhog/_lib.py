@@ -89,6 +89,8 @@ def lib() -> ctypes.CDLL:
     L.fhog_attn_fwd.argtypes = [POINTER(AttnArgs), c_void_p]
     L.fhog_attn_bwd.restype = c_int
     L.fhog_attn_bwd.argtypes = [POINTER(AttnArgs), c_void_p]
+    L.fhog_probe_mfma_rate.restype = c_int
+    L.fhog_probe_mfma_rate.argtypes = [c_void_p, c_int, c_int, c_int, POINTER(ctypes.c_double), c_void_p]
     if L.fhog_attn_args_size() != ctypes.sizeof(AttnArgs):
         raise RuntimeError("fhog_attn_args layout differs between libfhog_hip.so and the ctypes mirror")
     if L.fhog_bwdbwd_args_size() != ctypes.sizeof(BwdBwdArgs):

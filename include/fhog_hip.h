@@ -163,6 +163,13 @@ int fhog_attn_fwd(const fhog_attn_args* args, void* hip_stream);
    sweep for dK and dV), without the (batch, n_q, n_k) tensors. */
 int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream);
 
+/* Measurement aid (no counterpart in the reference): enqueue a loop of nothing but bf16 32x32x16 MFMAs on `blocks`
+   workgroups of 8 waves (one per CU fills the chip), `trips` x 32 MFMAs per wave, operands all zero (data_mode 0) or
+   random (data_mode 1). `out`: device buffer of blocks * 512 floats. Returns the FLOPs issued through *flops.
+   Timing it gives the MFMA rate the device sustains at the clock it holds for that operand data, the practical
+   ceiling next to the published peak. */
+int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream);
+
 /* Message for the last failing call on this thread ("" if none). */
 const char* fhog_last_error(void);
 

@@ -33,7 +33,8 @@ def test_header_symbols_exported(L):
     names = re.findall(r"^\s*(?:int|size_t|const char\*)\s+(fhog_\w+)\s*\(", header, flags=re.M)
     assert set(names) >= {"fhog_abi_version", "fhog_bwdbwd_args_size", "fhog_bwdbwd_workspace_bytes", "fhog_validate", "fhog_select_impl",
                           "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error",
-                          "fhog_attn_args_size", "fhog_attn_validate", "fhog_attn_fwd", "fhog_attn_bwd"}
+                          "fhog_attn_args_size", "fhog_attn_validate", "fhog_attn_fwd", "fhog_attn_bwd",
+                          "fhog_probe_mfma_rate"}
     for n in names:
         assert hasattr(L, n), n
 
@@ -135,6 +136,13 @@ def test_validate_rejects(L, mutate, code, word):
     # the compute entry points refuse the same way, before any launch
     assert L.fhog_bwdbwd(ctypes.byref(a), None) == code
     assert L.fhog_bwdbwd_pass(ctypes.byref(a), 1, None) == code
+
+
+def test_probe_rejects_bad_arguments(L):
+    flops = ctypes.c_double()
+    assert L.fhog_probe_mfma_rate(None, 256, 10, 0, ctypes.byref(flops), None) == -1
+    assert L.fhog_probe_mfma_rate(0x10000, 0, 10, 0, ctypes.byref(flops), None) == -2
+    assert L.fhog_probe_mfma_rate(0x10000, 256, 10, 2, ctypes.byref(flops), None) == -2
 
 
 def test_null_args(L):

@@ -303,6 +303,22 @@ def test_peak_memory_is_linear_in_n():
     assert sizes[8192] <= 4.2 * sizes[2048]
 
 
+def test_mfma_rate_probe_runs():
+    """The measurement aid of bench.py: launches, reports the FLOPs it issued, leaves finite sums."""
+    import ctypes
+    from fhog import _lib
+    L = _lib.lib()
+    out = torch.full((8 * 512,), float("nan"), device="cuda:0")
+    flops = ctypes.c_double()
+    for mode in (0, 1):
+        _lib.check(L.fhog_probe_mfma_rate(out.data_ptr(), 8, 100, mode, ctypes.byref(flops),
+                                          ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        assert flops.value == 8 * 8 * 100 * 32 * 32768
+        assert torch.isfinite(out).all()
+    assert out.abs().max() > 0   # random operands leave non-zero sums
+
+
 # ---------------------------------------------------------------- autograd chain
 @pytest.mark.parametrize("causal", [False, True])
 def test_autograd_chain_reaches_hip_double_backward(causal):
