@@ -77,7 +77,8 @@ struct TileVals {
 template <int D, int LEVEL, bool CAUSAL>
 __device__ inline TileVals tile_math(const float* Qs, const float* dOs, const float* ddQs, const float* Ks,
                                      const float* Vs, const float* ddKs, const float* ddVs, int lane, int q0,
-                                     int k0, int n_q, int n_k, float scale, float L, float dsum, float dd, float b) {
+                                     int k0, int n_q, int n_k, float scale, float L, float dsum, float dd, float b,
+                                     int mask_off, int window) {
   TileVals t;
   const f32x16_t zero = {0};
   f32x16_t s = mma_nt<D>(zero, Ks, Qs, lane);
@@ -95,7 +96,8 @@ __device__ inline TileVals tile_math(const float* Qs, const float* dOs, const fl
   for (int r = 0; r < 16; r++) {
     const int kj = k0 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
     bool valid = (qi < n_q) && (kj < n_k);
-    if (CAUSAL) valid = valid && (kj <= qi);
+    // band mask: key visible iff 0 <= (qi + mask_off) - kj < window (fhog/jax_refs/jax_impl.py:110-115)
+    if (CAUSAL) valid = valid && (kj <= qi + mask_off) && (qi + mask_off - kj < window);
     const float p = valid ? expf(s[r] * scale - L) : 0.f;
     const float ddsv = dds[r] * scale;
     t.p[r] = p;
@@ -212,9 +214,13 @@ __global__ void __launch_bounds__(64) q_sweep_fp32(Params p) {
     acc_ddo[cb] = f32x16_t{0};
   }
 
-  int k_end = p.n_k;
-  if (CAUSAL) k_end = min(p.n_k, q0 + TR);
-  for (int k0 = 0; k0 < k_end; k0 += TR) {
+  // key tiles that hold a visible key for some query of this tile
+  int k_begin = 0, k_end = p.n_k;
+  if (CAUSAL) {
+    k_end = min(p.n_k, q0 + TR + p.mask_off);
+    k_begin = max(0, q0 + p.mask_off - p.window + 1) / TR * TR;
+  }
+  for (int k0 = k_begin; k0 < k_end; k0 += TR) {
     __syncthreads();
     load_tile<T, D>(Ks, K, p.stride_kn, k0, p.n_k, lane);
     load_tile<T, D>(ddKs, ddK, p.stride_kn, k0, p.n_k, lane);
@@ -224,7 +230,7 @@ __global__ void __launch_bounds__(64) q_sweep_fp32(Params p) {
     }
     __syncthreads();
     TileVals t = tile_math<D, PASS, CAUSAL>(Qs, dOs, ddQs, Ks, Vs, ddKs, ddVs, lane, q0, k0, p.n_q, p.n_k, p.scale, L,
-                                            dsum, dd, b);
+                                            dsum, dd, b, p.mask_off, p.window);
     if (PASS == 1) red += t.dd_part;
     if (PASS == 2) red += t.b_part;
     if (PASS == 3) {
@@ -289,8 +295,13 @@ __global__ void __launch_bounds__(64) k_sweep_fp32(Params p) {
     acc_dv[cb] = f32x16_t{0};
   }
 
-  const int q_begin = CAUSAL ? k0 : 0;  // tiles are aligned: queries before k0 see none of these keys
-  for (int q0 = q_begin; q0 < p.n_q; q0 += TR) {
+  // query tiles that hold a query seeing some key of this tile: k - mask_off <= i < k - mask_off + window
+  int q_begin = 0, q_end = p.n_q;
+  if (CAUSAL) {
+    q_begin = max(0, k0 - p.mask_off) / TR * TR;
+    q_end = (int)min((int64_t)p.n_q, (int64_t)k0 + TR - 1 - p.mask_off + p.window);
+  }
+  for (int q0 = q_begin; q0 < q_end; q0 += TR) {
     __syncthreads();
     load_tile<T, D>(Qs, Q, p.stride_qn, q0, p.n_q, lane);
     load_tile<T, D>(dOs, dO, p.stride_qn, q0, p.n_q, lane);
@@ -304,7 +315,7 @@ __global__ void __launch_bounds__(64) k_sweep_fp32(Params p) {
     const float b = qok ? p.ws_b[row] : 0.f;
     __syncthreads();
     TileVals t = tile_math<D, 3, CAUSAL>(Qs, dOs, ddQs, Ks, Vs, ddKs, ddVs, lane, q0, k0, p.n_q, p.n_k, p.scale, L, dsum,
-                                         dd, b);
+                                         dd, b, p.mask_off, p.window);
     spill_tile(Wds, t.ds, lane);
     spill_tile(Wds2, t.ds2, lane);
     spill_tile(Wddp, t.ddp, lane);

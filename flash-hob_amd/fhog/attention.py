@@ -26,7 +26,7 @@ import ctypes
 import torch
 
 from . import _lib
-from .bwdbwd import flash_bwdbwd
+from .bwdbwd import flash_bwdbwd, mask_code
 
 _HIP_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
 _BLOCK_ELEMS = 1 << 26  # fp32 elements of one materialised (heads, rows, N_K) block (256 MiB)
@@ -41,14 +41,24 @@ def _blocks(batch: int, n_q: int, n_k: int):
             yield slice(b0, min(batch, b0 + heads)), slice(r0, min(n_q, r0 + rows))
 
 
-def _scores(q, k, scale, causal, r0):
+def _scores(q, k, scale, causal, r0, n_q=None, window=None):
+    """fp32 scores of query rows r0.. against all keys, masked entries at -inf."""
     s = torch.matmul(q.float(), k.float().transpose(-1, -2)) * scale
     if causal:
         n_r, n_k = s.shape[-2], s.shape[-1]
-        qi = torch.arange(r0, r0 + n_r, device=s.device)[:, None]
+        shift = (n_k - n_q) if causal == "bottom_right" else 0
+        qi = torch.arange(r0, r0 + n_r, device=s.device)[:, None] + shift
         kj = torch.arange(n_k, device=s.device)[None, :]
-        s = s.masked_fill(kj > qi, float("-inf"))
+        hidden = kj > qi
+        if window is not None:
+            hidden = hidden | (qi - kj >= window)
+        s = s.masked_fill(hidden, float("-inf"))
     return s
+
+
+def _plain_mask(causal, window, n_q, n_k) -> bool:
+    """No mask or the square causal mask without an effective window: what the 16-bit HIP kernels implement."""
+    return not causal or (n_q == n_k and (window is None or window >= n_k))
 
 
 def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
@@ -114,7 +124,8 @@ def _attention_backward_hip(q, k, v, o, do, L, scale, causal):
     return dq, dk, dv
 
 
-def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = False, *, use_hip: Optional[bool] = None):
+def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, window: Optional[int] = None,
+                      use_hip: Optional[bool] = None):
     """O (dtype of q) and fp32 L = logsumexp_j(scale q.k_j) for (batch, N, d) tensors.
 
     Takes the place of the reference's forward kernel outputs (``fhog/triton_flash.py:123-133``)
@@ -126,15 +137,15 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = Fal
     """
     if q.dim() == 4:
         B, H = q.shape[:2]
-        o, L = attention_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), scale, causal, use_hip=use_hip)
+        o, L = attention_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), scale, causal, window=window,
+                                 use_hip=use_hip)
         return o.view(q.shape), L.view(B, H, -1)
     batch, n_q, d = q.shape
     n_k = k.shape[1]
-    if causal and n_q != n_k:
-        raise ValueError("causal needs N_Q == N_K")
+    mask_code(causal, window, n_q, n_k)  # raises on an inapplicable mask
     scale = d ** -0.5 if scale is None else scale
     if use_hip is not False:
-        res = _attention_forward_hip(q, k, v, scale, causal)
+        res = _attention_forward_hip(q, k, v, scale, causal) if _plain_mask(causal, window, n_q, n_k) else None
         if res is not None:
             return res
         if use_hip:
@@ -142,7 +153,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal: bool = Fal
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
-        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start)
+        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start, n_q, window)
         lse = torch.logsumexp(s, dim=-1)
         p = torch.exp(s - lse[..., None])
         o[hs, rs] = torch.matmul(p, v[hs].float()).to(q.dtype)
@@ -156,13 +167,14 @@ def produce_L(Q, K, is_causal: bool = False):
     return attention_forward(Q, K, K, None, is_causal)[1]
 
 
-def attention_backward(q, k, v, o, do, L, scale: float, causal: bool, *, use_hip: Optional[bool] = None):
+def attention_backward(q, k, v, o, do, L, scale: float, causal, *, window: Optional[int] = None,
+                       use_hip: Optional[bool] = None):
     """First-order backward (dQ, dK, dV); the arithmetic of ``fhog/triton_flash.py:201-220`` without the
     (batch, N_Q, N_K) tensors. ``use_hip`` as in :func:`attention_forward`."""
     batch, n_q, d = q.shape
     n_k = k.shape[1]
     if use_hip is not False:
-        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal)
+        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal) if _plain_mask(causal, window, n_q, n_k) else None
         if res is not None:
             return res
         if use_hip:
@@ -172,7 +184,7 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal: bool, *, use_hip
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)
     for hs, rs in _blocks(batch, n_q, n_k):
         qf, dof = q[hs, rs].float(), do[hs, rs].float()
-        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start)
+        s = _scores(q[hs, rs], k[hs], scale, causal, rs.start, n_q, window)
         p = torch.exp(s - L[hs, rs].float()[..., None])
         dsum = (o[hs, rs].float() * dof).sum(-1, keepdim=True)
         dp = torch.matmul(dof, v[hs].float().transpose(-1, -2))
@@ -191,13 +203,14 @@ class AttnBwd(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, q, k, v, o, do, L, scale, causal):
+    def forward(ctx, q, k, v, o, do, L, scale, causal, window=None):
         ctx.save_for_backward(q, k, v, o, do, L)
         ctx.scale = scale
         ctx.causal = causal
+        ctx.window = window
         sq = q.shape
         f = (lambda t: t.flatten(0, 1)) if q.dim() == 4 else (lambda t: t)
-        dq, dk, dv = attention_backward(f(q), f(k), f(v), f(o), f(do), f(L), scale, causal)
+        dq, dk, dv = attention_backward(f(q), f(k), f(v), f(o), f(do), f(L), scale, causal, window=window)
         return dq.view(sq), dk.view(k.shape), dv.view(v.shape)
 
     @staticmethod
@@ -205,9 +218,9 @@ class AttnBwd(torch.autograd.Function):
     def backward(ctx, ddq, ddk, ddv):
         q, k, v, o, do, L = ctx.saved_tensors
         dq2, dk2, dv2, ddo = flash_bwdbwd(q, k, v, o, do, ddq.contiguous(), ddk.contiguous(), ddv.contiguous(), L,
-                                          ctx.scale, causal=ctx.causal)
+                                          ctx.scale, causal=ctx.causal, window=ctx.window)
         # O and L are caches of (q, k, v): the four results are already total derivatives.
-        return dq2, dk2, dv2, None, ddo, None, None, None
+        return dq2, dk2, dv2, None, ddo, None, None, None, None
 
 
 class FlashAttention(torch.autograd.Function):
@@ -215,21 +228,23 @@ class FlashAttention(torch.autograd.Function):
     ``FlashAttention2`` (``fhog/triton_flash.py:136-198``), twice differentiable."""
 
     @staticmethod
-    def forward(ctx, q, k, v, is_causal=False):
+    def forward(ctx, q, k, v, is_causal=False, window=None):
         scale = q.shape[-1] ** -0.5
-        o, L = attention_forward(q, k, v, scale, is_causal)
+        o, L = attention_forward(q, k, v, scale, is_causal, window=window)
         ctx.save_for_backward(q, k, v, o, L)
         ctx.is_causal = is_causal
+        ctx.window = window
         ctx.scale = scale
         return o
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, L = ctx.saved_tensors
-        dq, dk, dv = AttnBwd.apply(q, k, v, o, do.contiguous(), L, ctx.scale, ctx.is_causal)
-        return dq, dk, dv, None
+        dq, dk, dv = AttnBwd.apply(q, k, v, o, do.contiguous(), L, ctx.scale, ctx.is_causal, ctx.window)
+        return dq, dk, dv, None, None
 
 
-def attention(q, k, v, is_causal: bool = False):
-    """Twice-differentiable scaled-dot-product attention (scale = d^-1/2)."""
-    return FlashAttention.apply(q, k, v, is_causal)
+def attention(q, k, v, is_causal=False, window: Optional[int] = None):
+    """Twice-differentiable scaled-dot-product attention (scale = d^-1/2). ``is_causal``: False | True |
+    "bottom_right"; ``window``: sliding-window length on top of a causal mask."""
+    return FlashAttention.apply(q, k, v, is_causal, window)

@@ -44,7 +44,35 @@ def workspace_floats(batch: int, n_q: int) -> int:
     return _lib.lib().fhog_bwdbwd_workspace_bytes(batch, n_q) // 4
 
 
-def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, fused_stats=False) -> _lib.BwdBwdArgs:
+def mask_code(causal, window, n_q: int, n_k: int):
+    """(FHOG_MASK_* code, window) of the C ABI for the Python-level mask arguments.
+
+    ``causal``: False | True (top-left, N_Q == N_K) | "bottom_right" (key j visible iff j <= i + N_K - N_Q,
+    ``fhog/jax_refs/jax_impl.py:110-115``); ``window``: None or the sliding-window length in keys."""
+    if causal is None or causal is False or causal == 0:
+        if window is not None:
+            raise ValueError("a sliding window needs a causal mask")
+        return _lib.MASK_NONE, 0
+    if causal is True or causal == 1:
+        if n_q != n_k:
+            raise ValueError(f"causal needs N_Q == N_K, got {n_q} and {n_k} (causal='bottom_right' aligns the diagonal "
+                             "to the last key)")
+        code = _lib.MASK_TOP_LEFT
+    elif causal == "bottom_right":
+        if n_k < n_q:
+            raise ValueError(f"causal='bottom_right' needs N_K >= N_Q, got {n_k} and {n_q}")
+        code = _lib.MASK_BOTTOM_RIGHT
+    else:
+        raise ValueError(f"causal must be False, True or 'bottom_right', got {causal!r}")
+    if window is None:
+        return code, 0
+    if int(window) < 1:
+        raise ValueError(f"window must be >= 1, got {window}")
+    return code, int(window)
+
+
+def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, fused_stats=False,
+                window=None) -> _lib.BwdBwdArgs:
     a = _lib.BwdBwdArgs()
     a.q, a.k, a.v, a.o, a.dO = Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dO.data_ptr()
     a.ddq, a.ddk, a.ddv = ddQ.data_ptr(), ddK.data_ptr(), ddV.data_ptr()
@@ -57,14 +85,14 @@ def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws,
     a.stride_kb, a.stride_kn = K.stride(0), K.stride(1)
     a.scale = float(scale)
     a.dtype = _DTYPES[Q.dtype]
-    a.causal = int(bool(causal))
+    a.causal, a.window = mask_code(causal, window, Q.shape[1], K.shape[1])
     a.impl = impl
     a.schedule = 1 if fused_stats else 0
     return a
 
 
-def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = False, impl: Optional[str] = None,
-                 fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None):
+def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window: Optional[int] = None,
+                 impl: Optional[str] = None, fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None):
     """Flash Higher-Order-Gradients: VJP of the attention backward pass.
 
     Same positional signature and return order as the reference
@@ -79,8 +107,12 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
             (any other dtype is up-cast; the reference passes it in the input dtype,
             ``fhog/triton_flash.py:255-257``).
         scale: python float.
-        causal: keyword only; top-left mask, needs N_Q == N_K. (The reference has no causal
-            double-backward.)
+        causal: keyword only. True: top-left mask (key j visible to query i iff j <= i), needs N_Q == N_K.
+            "bottom_right": j <= i + N_K - N_Q, needs N_K >= N_Q. (The reference's Triton path has no causal
+            double-backward; its JAX specification has the bottom-right form, ``fhog/jax_refs/jax_impl.py:110-115``.)
+        window: sliding-window length in keys on top of a causal mask (same function of the specification):
+            only the ``window`` most recent visible keys stay visible. The 16-bit MFMA kernels take no mask or
+            the plain square causal mask; other masks run on the fp32-MFMA kernels.
         impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the 16-bit MFMA kernels ("bf16": products
             in the tensor type, bf16 or fp16) for 16-bit tensors whose shape they support, the fp32-MFMA kernels
             otherwise.
@@ -124,8 +156,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
         raise ValueError(f"L has {L.numel()} elements, expected batch*N_Q = {batch * n_q}")
     if d not in (32, 64, 128):
         raise ValueError(f"head dim {d} not supported (32, 64 or 128)")
-    if causal and n_q != n_k:
-        raise ValueError(f"causal needs N_Q == N_K, got {n_q} and {n_k}")
+    mask_code(causal, window, n_q, n_k)  # raises on an inapplicable mask
     if not Q.is_cuda:
         raise ValueError("flash_bwdbwd runs on the GPU only: tensors must be on a ROCm device (there is no CPU path)")
     lse = L.reshape(batch, n_q)
@@ -142,7 +173,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal: bool = Fals
         dv2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
         ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
         args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl],
-                           (dq2, dk2, dv2, ddo), ws, fused_stats)
+                           (dq2, dk2, dv2, ddo), ws, fused_stats, window)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         L_ = _lib.lib()
         if only_pass is None:
@@ -165,7 +196,8 @@ class BwdBwdPlan:
     For benchmark loops and per-pass profiling; ``flash_bwdbwd`` is the drop-in entry point.
     """
 
-    def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, impl=None, fused_stats=False):
+    def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window=None, impl=None,
+                 fused_stats=False):
         ts = [_flatten(t, "tensor") for t in (Q, K, V, O, dO, ddQ, ddK, ddV)]
         q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = ts
         q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
@@ -175,7 +207,7 @@ class BwdBwdPlan:
         self.keep = (q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse)
         self.outs = (torch.empty_like(q3), torch.empty_like(k3), torch.empty_like(v3), torch.empty_like(q3))
         self.ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
-        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws, fused_stats)
+        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws, fused_stats, window)
         self.lib = _lib.lib()
         _lib.check(self.lib.fhog_validate(ctypes.byref(self.args)))
         self.impl = self.lib.fhog_select_impl(ctypes.byref(self.args))

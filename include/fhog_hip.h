@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FHOG_ABI_VERSION 1
+#define FHOG_ABI_VERSION 2
 
 /* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
 #define FHOG_DTYPE_BF16 0
@@ -42,7 +42,8 @@ extern "C" {
 #define FHOG_E_DTYPE (-3)     /* unknown dtype */
 #define FHOG_E_STRIDE (-4)    /* stride smaller than the row / not a multiple of the vector width */
 #define FHOG_E_ALIGN (-5)     /* pointer not 16-byte aligned */
-#define FHOG_E_CAUSAL (-6)    /* causal with n_q != n_k */
+#define FHOG_E_CAUSAL (-6)    /* mask not applicable: top-left causal with n_q != n_k, bottom-right with n_k < n_q,
+                                 a window without a causal mask, or a mask the forced kernel family does not take */
 #define FHOG_E_PASS (-7)      /* unknown pass id */
 #define FHOG_E_LAUNCH (-8)    /* HIP reported an error at launch */
 #define FHOG_E_SCALE (-9)     /* scale is not finite */
@@ -61,6 +62,14 @@ extern "C" {
 #define FHOG_IMPL_FP32 1   /* force the fp32-MFMA kernels (any dtype; every intermediate in fp32) */
 #define FHOG_IMPL_BF16 2   /* force the 16-bit MFMA kernels (bf16 or fp16 tensors, products in the tensor type);
                               error if the shape/dtype does not fit */
+
+/* masks (fhog_bwdbwd_args.causal). With a window W > 0 key j is visible to query i iff 0 <= i' - j < W, where i' = i
+   (top-left) or i' = i + n_k - n_q (bottom-right: fhog/jax_refs/jax_impl.py:110-115); W = 0 means no window.
+   The 16-bit MFMA kernels take FHOG_MASK_NONE and the plain square causal mask; every other mask runs on the
+   fp32-MFMA kernels. */
+#define FHOG_MASK_NONE 0
+#define FHOG_MASK_TOP_LEFT 1     /* j <= i; needs n_q == n_k (fhog/triton_flash.py:86-92) */
+#define FHOG_MASK_BOTTOM_RIGHT 2 /* j <= i + n_k - n_q; needs n_k >= n_q, so that every query sees a key */
 
 /* pass schedules of fhog_bwdbwd (fhog_bwdbwd_args.schedule) */
 #define FHOG_SCHEDULE_FOUR_PASS 0   /* the reference's schedule: d, then dd, b, dQ2+ddO, dK2+dV2 as four sweeps
@@ -92,9 +101,10 @@ typedef struct fhog_bwdbwd_args {
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   float scale;
   int32_t dtype;  /* FHOG_DTYPE_* */
-  int32_t causal; /* 0 | 1 (top-left mask: key j visible to query i iff j <= i; needs n_q == n_k) */
+  int32_t causal; /* FHOG_MASK_* */
   int32_t impl;   /* FHOG_IMPL_* */
   int32_t schedule; /* FHOG_SCHEDULE_* */
+  int64_t window; /* sliding window length in keys, 0 = none; needs a causal mask */
 } fhog_bwdbwd_args;
 
 /* Version of this header the library was built from. */

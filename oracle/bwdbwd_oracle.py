@@ -18,10 +18,11 @@ Two independent statements of the same function live here:
   not share a single formula with :func:`closed_form`.  This is the parity
   definition of the build (fp32 on the GPU tier, fp64 on the CPU tier).
 
-Causal convention: top-left, ``P_ij = 0`` for ``j > i`` (what
+Mask conventions: ``causal=True`` is top-left, ``P_ij = 0`` for ``j > i`` (what
 ``fhog/triton_flash.py:86-92`` and ``F.scaled_dot_product_attention(is_causal=True)``
-use).  For ``N_Q == N_K`` this equals the bottom-right mask of
-``fhog/jax_refs/jax_impl.py:110-115``.
+use).  ``causal="bottom_right"`` with an optional ``window`` is the mask of
+``fhog/jax_refs/jax_impl.py:110-115`` (key j visible iff ``0 <= i + N_K - N_Q - j < window``);
+for ``N_Q == N_K`` and no window the two are the same.
 
 Pinning status (tests/test_oracle.py):
   closed_form          pinned: == autograd (fp64, <=1e-10), == reference golden
@@ -32,6 +33,11 @@ Pinning status (tests/test_oracle.py):
   causal, d=128, N>256, fp32 inputs: no reference-held vector exists (the
   reference implements none of them); pinned by autograd == closed_form and the
   mathematical checks only.
+  bottom-right / sliding-window masks: no reference-held vector either; pinned by
+  closed_form == autograd == brute force on the same mask, by the mask itself
+  against the index formula of jax_impl.py:110-115, and by the reductions to known
+  cases (window >= N: plain causal; N_Q == N_K: top-left; window = 1: one key per
+  query, for which every gradient through the soft-max vanishes).
 """
 from __future__ import annotations
 
@@ -51,12 +57,28 @@ __all__ = [
 ]
 
 
-def _mask(n_q: int, n_k: int) -> np.ndarray:
-    """Top-left causal mask: True where key j may be attended by query i."""
-    return np.arange(n_q)[:, None] >= np.arange(n_k)[None, :]
+def _mask(n_q: int, n_k: int, causal=True, window: Optional[int] = None) -> Optional[np.ndarray]:
+    """Visibility mask: True where key j may be attended by query i; None when nothing is masked.
+
+    ``causal``: False | True (top-left: j <= i) | "bottom_right" (j <= i + N_K - N_Q, the mask of
+    ``fhog/jax_refs/jax_impl.py:110-115``).  ``window`` adds the sliding-window bound of the same
+    function: (shifted i) - j < window.
+    """
+    if not causal:
+        if window is not None:
+            raise ValueError("a sliding window needs a causal mask")
+        return None
+    if causal not in (True, "bottom_right"):
+        raise ValueError(f"unknown mask {causal!r}")
+    qi = np.arange(n_q)[:, None] + ((n_k - n_q) if causal == "bottom_right" else 0)
+    kj = np.arange(n_k)[None, :]
+    m = qi >= kj
+    if window is not None:
+        m &= (qi - kj) < window
+    return m
 
 
-def forward_o_lse(q, k, v, scale: float, causal: bool = False):
+def forward_o_lse(q, k, v, scale: float, causal=False, window: Optional[int] = None):
     """Materialised forward in float64: returns (O, L) with L = logsumexp_j(scale q.k).
 
     ``L`` is what ``fhog/triton_flash.py:252-258`` (``produce_L``) and the forward
@@ -67,8 +89,9 @@ def forward_o_lse(q, k, v, scale: float, causal: bool = False):
     k = np.asarray(k, dtype=np.float64)
     v = np.asarray(v, dtype=np.float64)
     s = scale * np.einsum("...id,...jd->...ij", q, k)
-    if causal:
-        s = np.where(_mask(q.shape[-2], k.shape[-2]), s, -np.inf)
+    m_ = _mask(q.shape[-2], k.shape[-2], causal, window)
+    if m_ is not None:
+        s = np.where(m_, s, -np.inf)
     m = s.max(axis=-1, keepdims=True)
     e = np.exp(s - m)
     l = e.sum(axis=-1, keepdims=True)
@@ -77,17 +100,18 @@ def forward_o_lse(q, k, v, scale: float, causal: bool = False):
     return o, lse
 
 
-def first_backward(q, k, v, do, scale: float, causal: bool = False):
+def first_backward(q, k, v, do, scale: float, causal=False, window: Optional[int] = None):
     """Materialised first-order attention backward (dQ, dK, dV) in float64.
 
     Same arithmetic as ``fhog/triton_flash.py:201-220``; used by the adjoint test.
     """
     q, k, v, do = (np.asarray(t, dtype=np.float64) for t in (q, k, v, do))
-    o, lse = forward_o_lse(q, k, v, scale, causal)
+    o, lse = forward_o_lse(q, k, v, scale, causal, window)
     s = scale * np.einsum("...id,...jd->...ij", q, k)
     p = np.exp(s - lse[..., None])
-    if causal:
-        p = np.where(_mask(q.shape[-2], k.shape[-2]), p, 0.0)
+    m_ = _mask(q.shape[-2], k.shape[-2], causal, window)
+    if m_ is not None:
+        p = np.where(m_, p, 0.0)
     d = np.einsum("...id,...id->...i", o, do)
     dp = np.einsum("...id,...jd->...ij", do, v)
     ds = scale * p * (dp - d[..., None])
@@ -97,8 +121,9 @@ def first_backward(q, k, v, do, scale: float, causal: bool = False):
     return dq, dk, dv
 
 
-def closed_form(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False,
-                o: Optional[np.ndarray] = None, lse: Optional[np.ndarray] = None) -> Dict[str, np.ndarray]:
+def closed_form(q, k, v, do, ddq, ddk, ddv, scale: float, causal=False,
+                o: Optional[np.ndarray] = None, lse: Optional[np.ndarray] = None,
+                window: Optional[int] = None) -> Dict[str, np.ndarray]:
     """Materialised double-backward in float64.
 
     Inputs broadcast over leading dims; q, do, ddq: (..., N_Q, d); k, v, ddk, ddv: (..., N_K, d).
@@ -109,7 +134,7 @@ def closed_form(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False,
     """
     q, k, v, do, ddq, ddk, ddv = (np.asarray(t, dtype=np.float64) for t in (q, k, v, do, ddq, ddk, ddv))
     if o is None or lse is None:
-        o_x, lse_x = forward_o_lse(q, k, v, scale, causal)
+        o_x, lse_x = forward_o_lse(q, k, v, scale, causal, window)
         o = o_x if o is None else np.asarray(o, dtype=np.float64)
         lse = lse_x if lse is None else np.asarray(lse, dtype=np.float64)
     else:
@@ -118,8 +143,9 @@ def closed_form(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False,
 
     s = scale * np.einsum("...id,...jd->...ij", q, k)            # jax_impl.py:314-319
     p = np.exp(s - lse[..., None])                               # jax_impl.py:326
-    if causal:
-        p = np.where(_mask(q.shape[-2], k.shape[-2]), p, 0.0)   # jax_impl.py:321-324
+    m_ = _mask(q.shape[-2], k.shape[-2], causal, window)
+    if m_ is not None:
+        p = np.where(m_, p, 0.0)   # jax_impl.py:321-324
     dp = np.einsum("...id,...jd->...ij", do, v)                  # jax_impl.py:328
     dds = scale * (np.einsum("...id,...jd->...ij", ddq, k)
                    + np.einsum("...id,...jd->...ij", q, ddk))    # jax_impl.py:329
@@ -138,8 +164,8 @@ def closed_form(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False,
     return dict(dq2=dq2, dk2=dk2, dv2=dv2, ddo=ddo, L=lse, d=d, dd=dd, b=b, o=o)
 
 
-def autograd_double_backward(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False,
-                             dtype: torch.dtype = torch.float64, head_chunk: int = 1):
+def autograd_double_backward(q, k, v, do, ddq, ddk, ddv, scale: float, causal=False,
+                             dtype: torch.dtype = torch.float64, head_chunk: int = 1, window: Optional[int] = None):
     """Double backward through materialised softmax attention with torch autograd.
 
     Accepts torch tensors or numpy arrays of shape (batch, N, d) (or (N, d)); loops
@@ -156,9 +182,9 @@ def autograd_double_backward(q, k, v, do, ddq, ddk, ddv, scale: float, causal: b
     batch, n_q, _ = q_.shape
     n_k = k_.shape[1]
     outs = [torch.empty_like(q_), torch.empty_like(k_), torch.empty_like(v_), torch.empty_like(do_)]
-    mask = None
-    if causal:
-        mask = torch.ones(n_q, n_k, dtype=torch.bool, device=q_.device).tril()
+    mask = _mask(n_q, n_k, causal, window)
+    if mask is not None:
+        mask = torch.from_numpy(mask).to(q_.device)
     for b0 in range(0, batch, head_chunk):
         sl = slice(b0, min(batch, b0 + head_chunk))
         qh = q_[sl].detach().clone().requires_grad_(True)
@@ -179,7 +205,7 @@ def autograd_double_backward(q, k, v, do, ddq, ddk, ddv, scale: float, causal: b
     return tuple(outs)
 
 
-def brute_force(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False):
+def brute_force(q, k, v, do, ddq, ddk, ddv, scale: float, causal=False, window: Optional[int] = None):
     """Scalar-loop evaluation for tiny single-head inputs (N <= 8, d <= 4).
 
     Written index by index from the handwritten equations
@@ -199,7 +225,9 @@ def brute_force(q, k, v, do, ddq, ddk, ddv, scale: float, causal: bool = False):
             for c in range(dh):
                 sij += q[i, c] * k[j, c]
             srow.append(scale * sij)
-        allowed = [j for j in range(nk) if (not causal) or j <= i]
+        shift = (nk - nq) if causal == "bottom_right" else 0
+        allowed = [j for j in range(nk)
+                   if (not causal) or (j <= i + shift and (window is None or i + shift - j < window))]
         mx = max(srow[j] for j in allowed)
         z = sum(math.exp(srow[j] - mx) for j in allowed)
         for j in allowed:

@@ -27,10 +27,11 @@ def make_case(batch, n_q, n_k, d, dtype, seed, grad_std=1.0, k_row_scale=False, 
     return {n: t.to(dtype).to(device) for n, t in x.items()}
 
 
-def with_caches(x, scale, causal):
+def with_caches(x, scale, causal, window=None):
     """Add O (input dtype) and fp32 L from an fp32 forward on the rounded inputs."""
     import fhog
-    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, use_hip=False)  # fp32 forward on the rounded inputs
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, window=window,
+                                  use_hip=False)  # fp32 forward on the rounded inputs
     return dict(x, O=o, L=L)
 
 
@@ -47,9 +48,9 @@ def reference_fp32_gpu(x, scale, causal, heads=None, head_chunk=1):
                                     sel(x["ddV"]), scale, causal, dtype=torch.float32, head_chunk=head_chunk)
 
 
-def reference_fp64_cpu(x, scale, causal):
+def reference_fp64_cpu(x, scale, causal, window=None):
     c = {n: t.detach().double().cpu().numpy() for n, t in x.items()}
-    return closed_form(c["Q"], c["K"], c["V"], c["dO"], c["ddQ"], c["ddK"], c["ddV"], scale, causal)
+    return closed_form(c["Q"], c["K"], c["V"], c["dO"], c["ddQ"], c["ddK"], c["ddV"], scale, causal, window=window)
 
 
 def errors(outs, refs):

@@ -56,7 +56,7 @@ def _header_fields(struct_name):
 def test_struct_mirror_matches_header():
     from fhog import _lib
     assert _header_fields("fhog_bwdbwd_args") == [f[0] for f in _lib.BwdBwdArgs._fields_]
-    assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 200
+    assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 208
     assert _header_fields("fhog_attn_args") == [f[0] for f in _lib.AttnArgs._fields_]
     assert ctypes.sizeof(_lib.AttnArgs) == _lib.lib().fhog_attn_args_size() == 160
 
@@ -97,7 +97,7 @@ def test_attn_validate(L, mutate, backward, code, word):
 
 
 def test_version_and_workspace(L):
-    assert L.fhog_abi_version() == 1
+    assert L.fhog_abi_version() == 2
     assert L.fhog_bwdbwd_workspace_bytes(32, 4096) == 3 * 32 * 4096 * 4
     assert L.fhog_bwdbwd_workspace_bytes(-1, 5) == 0
 
@@ -124,8 +124,12 @@ def test_validate_accepts_good(L):
     (lambda a: setattr(a, "stride_kn", 68), -4, "multiples"),
     (lambda a: setattr(a, "stride_qb", 64), -4, "batch stride"),
     (lambda a: setattr(a, "k", 0x20004), -5, "aligned"),
-    (lambda a: setattr(a, "causal", 1), -6, "causal"),
-    (lambda a: setattr(a, "causal", 2), -6, "causal"),
+    (lambda a: setattr(a, "causal", 1), -6, "top-left"),          # n_q != n_k
+    (lambda a: setattr(a, "causal", 3), -6, "causal"),
+    (lambda a: (setattr(a, "causal", 2), setattr(a, "n_k", 128), setattr(a, "stride_kb", 128 * 64)), -6, "bottom-right"),
+    (lambda a: setattr(a, "window", 16), -6, "window needs"),
+    (lambda a: (setattr(a, "causal", 2), setattr(a, "window", -1)), -6, "window"),
+    (lambda a: (setattr(a, "causal", 2), setattr(a, "impl", 2)), -6, "impl=bf16 takes"),
     (lambda a: setattr(a, "scale", float("nan")), -9, "scale"),
 ])
 def test_validate_rejects(L, mutate, code, word):
@@ -143,6 +147,20 @@ def test_probe_rejects_bad_arguments(L):
     assert L.fhog_probe_mfma_rate(None, 256, 10, 0, ctypes.byref(flops), None) == -1
     assert L.fhog_probe_mfma_rate(0x10000, 0, 10, 0, ctypes.byref(flops), None) == -2
     assert L.fhog_probe_mfma_rate(0x10000, 256, 10, 2, ctypes.byref(flops), None) == -2
+
+
+def test_masks_select_the_kernel_family(L):
+    a = good_args()                       # bf16, 256 x 512, d = 64: shape fits the 16-bit kernels
+    assert L.fhog_select_impl(ctypes.byref(a)) == 2
+    a.causal = 2                          # bottom-right on a rectangular problem: fp32-MFMA kernels
+    assert L.fhog_validate(ctypes.byref(a)) == 0
+    assert L.fhog_select_impl(ctypes.byref(a)) == 1
+    a.n_k, a.stride_kb = 256, 256 * 64    # square: bottom-right == top-left, 16-bit kernels again
+    assert L.fhog_select_impl(ctypes.byref(a)) == 2
+    a.window = 64
+    assert L.fhog_select_impl(ctypes.byref(a)) == 1
+    a.window = 256                        # a window that hides nothing
+    assert L.fhog_select_impl(ctypes.byref(a)) == 2
 
 
 def test_null_args(L):
@@ -173,7 +191,13 @@ def test_python_wrapper_errors():
     with pytest.raises(ValueError):
         fhog.flash_bwdbwd(q, k, k, q, q, q, k, t(2, 64, 64), L, 0.125)
     with pytest.raises(ValueError):
-        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125, causal=True)
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125, causal=True)      # top-left needs N_Q == N_K
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(k, q, q, k, k, k, q, q, torch.zeros(2, 128), 0.125, causal="bottom_right")  # N_K < N_Q
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125, window=8)         # window without a causal mask
+    with pytest.raises(ValueError):
+        fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, L, 0.125, causal="upper")
     with pytest.raises(ValueError):
         fhog.flash_bwdbwd(q, k, k, q, q, q, k, k, torch.zeros(2, 63), 0.125)
     with pytest.raises(ValueError, match="GPU only"):

@@ -25,7 +25,7 @@ def _dev():
 def test_library_is_the_hip_one():
     from fhog import _lib
     assert _lib.LIB_PATH.exists()
-    assert _lib.lib().fhog_abi_version() == 1
+    assert _lib.lib().fhog_abi_version() == _lib.ABI_VERSION
 
 
 # ---------------------------------------------------------------- reference golden tensors
@@ -94,6 +94,43 @@ def test_fp32_family_ragged(shape, causal, dtype):
     stat_tol = 1e-4 if dtype == torch.float32 else 5e-3   # bf16: O is rounded before d = rowsum(O*dO)
     for got, name in zip(outs[4], ("d", "dd", "b")):
         assert normalised_max_error(got, ref[name]) < stat_tol, name
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [("bottom_right", None, 100, 177), ("bottom_right", 40, 100, 177), (True, 33, 160, 160),
+                                  ("bottom_right", 1, 64, 96), ("bottom_right", 500, 31, 31), (True, 7, 256, 256)])
+def test_bottom_right_and_sliding_window_masks(mask, dtype):
+    """The masks of the reference's specification (fhog/jax_refs/jax_impl.py:110-115), which its Triton path lacks:
+    bottom-right alignment for N_Q != N_K and a sliding window; they run on the fp32-MFMA kernels."""
+    causal, window, n_q, n_k = mask
+    d = 64
+    x = make_case(2, n_q, n_k, d, dtype, seed=15)
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal, window)
+    outs = run_fhog(x, scale, causal, window=window, return_stats=True)
+    ref = reference_fp64_cpu(x, scale, causal, window)
+    e = errors(outs[:4], [ref[n] for n in NAMES])
+    assert max(e.values()) < TOL[dtype], e
+    stat_tol = 1e-4 if dtype == torch.float32 else 5e-3
+    for got, name in zip(outs[4], ("d", "dd", "b")):
+        assert normalised_max_error(got, ref[name]) < stat_tol, name
+
+
+def test_masks_that_hide_nothing_more_take_the_16_bit_kernels():
+    """Square bottom-right == top-left, and a window as long as the sequence: same kernels, same bits."""
+    from fhog import BwdBwdPlan
+    x = with_caches(make_case(2, 256, 256, 64, torch.bfloat16, seed=16, grad_std=0.1), 0.125, True)
+    base = run_fhog(x, 0.125, True)
+    for kw in (dict(causal="bottom_right"), dict(causal=True, window=256), dict(causal="bottom_right", window=4096)):
+        plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125, **kw)
+        assert plan.impl == 2
+        outs = plan.run()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, base):
+            assert torch.equal(a, b)
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125,
+                      causal=True, window=64)
+    assert plan.impl == 1
 
 
 def test_strided_and_4d_inputs():
@@ -317,6 +354,29 @@ def test_mfma_rate_probe_runs():
         assert flops.value == 8 * 8 * 100 * 32 * 32768
         assert torch.isfinite(out).all()
     assert out.abs().max() > 0   # random operands leave non-zero sums
+
+
+def test_autograd_chain_with_a_sliding_window():
+    """attention(..., 'bottom_right', window) twice differentiated against torch autograd on the same mask."""
+    import fhog
+    g = torch.Generator().manual_seed(9)
+    mk = lambda *s: torch.randn(*s, generator=g).cuda()
+    q, k, v, w = mk(2, 96, 64), mk(2, 160, 64), mk(2, 160, 64), mk(2, 96, 64)
+    qi = torch.arange(96, device="cuda")[:, None] + 64
+    kj = torch.arange(160, device="cuda")[None, :]
+    visible = (kj <= qi) & (qi - kj < 50)
+
+    def penalty(attn):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = attn(qq, kk, vv)
+        gq, gk, gv = torch.autograd.grad((out * w).sum(), (qq, kk, vv), create_graph=True)
+        loss = gq.square().sum() + (gk * gv).sum()
+        return torch.autograd.grad(loss, (qq, kk, vv))
+
+    ours = penalty(lambda a, b, c: fhog.attention(a, b, c, "bottom_right", 50))
+    ref = penalty(lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(a, b, c, attn_mask=visible))
+    for a, b in zip(ours, ref):
+        assert normalised_max_error(a, b) < 1e-4
 
 
 # ---------------------------------------------------------------- autograd chain

@@ -186,3 +186,54 @@ def test_autograd_fp32_head_chunking_matches_fp64():
     a32 = autograd_double_backward(*args, dtype=torch.float32, head_chunk=2)
     for u, w in zip(a32, a64):
         assert normalised_max_error(u, w) < 1e-5
+
+
+# ---------------------------------------------------------------- bottom-right and sliding-window masks
+def test_mask_follows_the_reference_index_formula():
+    """The mask itself against fhog/jax_refs/jax_impl.py:110-115, index by index."""
+    from oracle.bwdbwd_oracle import _mask
+    for n_q, n_k, w in [(3, 5, None), (4, 4, 2), (2, 7, 3), (5, 5, 1), (6, 9, 100)]:
+        m = _mask(n_q, n_k, "bottom_right", w)
+        for i in range(n_q):
+            for j in range(n_k):
+                qi = i + n_k - n_q
+                assert bool(m[i, j]) == (qi >= j and (w is None or qi - j < w)), (n_q, n_k, w, i, j)
+        assert m.any(axis=1).all()   # with N_K >= N_Q every query sees at least one key
+    assert np.array_equal(_mask(6, 6, "bottom_right"), _mask(6, 6, True))
+    assert np.array_equal(_mask(6, 6, True, 100), _mask(6, 6, True))
+    assert _mask(4, 9, False) is None
+
+
+@pytest.mark.parametrize("spec", [("bottom_right", None, 12, 20), ("bottom_right", 5, 12, 20), (True, 4, 16, 16),
+                                  ("bottom_right", 7, 16, 16)])
+def test_band_masks_closed_form_equals_autograd_and_brute_force(spec):
+    causal, window, n_q, n_k = spec
+    rng = np.random.default_rng(5)
+    x = rand_inputs(rng, n_q, n_k, 8, batch=(2,))
+    scale = 8 ** -0.5
+    cf = closed_form(**x, scale=scale, causal=causal, window=window)
+    ag = autograd_double_backward(x["q"], x["k"], x["v"], x["do"], x["ddq"], x["ddk"], x["ddv"], scale, causal,
+                                  window=window)
+    for n, a in zip(NAMES, ag):
+        assert normalised_max_error(cf[n], a) < 1e-10, n
+    y = rand_inputs(rng, 4, 6 if causal == "bottom_right" else 4, 2)
+    w_small = None if window is None else 2
+    cf = closed_form(**y, scale=0.7, causal=causal, window=w_small)
+    bf = brute_force(y["q"], y["k"], y["v"], y["do"], y["ddq"], y["ddk"], y["ddv"], 0.7, causal, w_small)
+    for n, b in zip(NAMES, bf):
+        np.testing.assert_allclose(cf[n], b, rtol=1e-11, atol=1e-12, err_msg=n)
+
+
+def test_band_mask_reductions_to_known_cases():
+    rng = np.random.default_rng(6)
+    x = rand_inputs(rng, 10, 10, 4)
+    base = closed_form(**x, scale=0.5, causal=True)
+    for other in (closed_form(**x, scale=0.5, causal="bottom_right"), closed_form(**x, scale=0.5, causal=True, window=10)):
+        for n in NAMES:
+            np.testing.assert_allclose(other[n], base[n], rtol=0, atol=0)
+    # window 1: every query sees exactly one key, P = 1 there: no gradient flows through the soft-max
+    one = closed_form(**x, scale=0.5, causal=True, window=1)
+    np.testing.assert_allclose(one["dq2"], 0, atol=1e-12)
+    np.testing.assert_allclose(one["dk2"], 0, atol=1e-12)
+    np.testing.assert_allclose(one["dv2"], 0, atol=1e-12)
+    np.testing.assert_allclose(one["ddo"], x["ddv"], atol=1e-12)   # O_i = V_i, so ddO_i = ddV_i
