@@ -340,6 +340,43 @@ def test_peak_memory_is_linear_in_n():
     assert sizes[8192] <= 4.2 * sizes[2048]
 
 
+def test_hip_graph_capture_and_replay():
+    """The library only enqueues kernels on the caller's stream: a captured call replays to the same bits, also after
+    the inputs changed in place and with eager work in between."""
+    from fhog import BwdBwdPlan
+    x = with_caches(make_case(4, 512, 512, 128, torch.bfloat16, seed=17, grad_std=0.1), 128 ** -0.5, True)
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 128 ** -0.5, causal=True)
+    eager = [t.clone() for t in plan.run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan.run()                       # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        plan.run()
+    for rep in range(3):
+        for o in plan.outs:
+            o.fill_(float("nan"))
+        plan.ws.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(plan.outs, eager):
+            assert torch.equal(a, b), rep
+        _ = (x["Q"].float() @ x["K"].float().transpose(-1, -2)).sum().item()   # unrelated eager work between replays
+    # the graph reads the plan's input buffers: new values in place, same graph
+    q_in = plan.keep[7]                  # ddV as the plan holds it
+    q_in.mul_(2.0)
+    graph.replay()
+    torch.cuda.synchronize()
+    fresh = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], q_in, x["L"], 128 ** -0.5, causal=True)
+    want = fresh.run()
+    torch.cuda.synchronize()
+    for a, b in zip(plan.outs, want):
+        assert torch.equal(a, b)
+
+
 def test_mfma_rate_probe_runs():
     """The measurement aid of bench.py: launches, reports the FLOPs it issued, leaves finite sums."""
     import ctypes
