@@ -55,6 +55,12 @@ __device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int
   }
 }
 
+// registers 4g..4g+3 only (one ds_write_b64), so that the hand-off writes can be spread over the stream
+__device__ __forceinline__ void sop_write_group(char* tile, uint32_t lo, uint32_t hi, int g, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+  *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = u32x2_t{lo, hi};
+}
+
 template <bool F16, int D>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
                                           const bf16x8_t* dOb, int lane, int q_idx, int k_base, bool mask,
@@ -103,6 +109,13 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
         us[r] = u0 * scale;
         us[r + 1] = u1 * scale;
       }
+      // a group of four registers is complete every 4 / EPK steps: hand it off right away, so that the writes
+      // travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
+      if ((EPK * (kk + 1)) % 4 == 0) {
+#pragma unroll
+        for (int g = (EPK * kk) / 4; g < (EPK * (kk + 1)) / 4; g++)
+          sop_write_group(sop + 0 * SOP_TILE, pk_ds[2 * g], pk_ds[2 * g + 1], g, lane);
+      }
     } else {
       e = mfma<F16>(a[c], dOb[kk], e);
 #pragma unroll
@@ -112,12 +125,16 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
         vv[r] = pv[r] * __builtin_fmaf(dds[r], us[r], -vv[r]);              // z
         vv[r + 1] = pv[r + 1] * __builtin_fmaf(dds[r + 1], us[r + 1], -vv[r + 1]);
       }
+      if ((EPK * (kk + 1)) % 4 == 0) {
+#pragma unroll
+        for (int g = (EPK * kk) / 4; g < (EPK * (kk + 1)) / 4; g++) {
+          sop_write_group(sop + 2 * SOP_TILE, pk_ddp[2 * g], pk_ddp[2 * g + 1], g, lane);
+          sop_write_group(sop + 3 * SOP_TILE, pk_p[2 * g], pk_p[2 * g + 1], g, lane);
+        }
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  sop_write_pk(sop + 0 * SOP_TILE, pk_ds, lane);
-  sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, lane);
-  sop_write_pk(sop + 3 * SOP_TILE, pk_p, lane);
 #pragma unroll
   for (int r = 0; r < 16; r += 2)
     pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
