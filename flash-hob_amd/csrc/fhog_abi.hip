@@ -65,7 +65,7 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->impl == FHOG_IMPL_BF16) {
     if (a->dtype == FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "impl=bf16 needs bf16 or fp16 tensors");
     if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
-      return fail(FHOG_E_SHAPE, "impl=bf16 needs d in {64,128} and n_q, n_k multiples of 128");
+      return fail(FHOG_E_SHAPE, "impl=bf16 needs d in {64,128}");
     if (!plain_mask(a)) return fail(FHOG_E_CAUSAL, "impl=bf16 takes no mask or the square causal mask without a window");
   }
   return FHOG_OK;
@@ -147,7 +147,7 @@ int validate_attn(const fhog_attn_args* a, int backward) {
   if (a->causal != 0 && a->causal != 1) return fail(FHOG_E_CAUSAL, "causal must be 0 or 1");
   if (a->causal && a->n_q != a->n_k) return fail(FHOG_E_CAUSAL, "causal needs n_q == n_k");
   if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
-    return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128} and n_q, n_k multiples of 128");
+    return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128}");
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
   if (a->stride_qn % 8 || a->stride_kn % 8 || a->stride_qb % 8 || a->stride_kb % 8)

@@ -87,16 +87,17 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
-  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[2] = {(const __bf16*)p.k + koff, (const __bf16*)p.v + koff};
 
   bf16x8_t Qb[KK];
-  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
+  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
   wait_vm0();
   const float c_scale_log2 = p.scale * kLog2e;
 
@@ -113,12 +114,13 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
 #pragma unroll
   for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
 
-  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  const int k_tiles = (p.n_k + TS - 1) / TS;
+  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
 #pragma unroll
-  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave);
+  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
   dma_wait();
   __syncthreads();
 
@@ -127,9 +129,13 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
 #pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
+    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key);
+    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
+    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
+    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
     if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
       const char* stage = smem + (j & 1) * STAGE;
       f32x16_t s[1] = {f32x16_t{0}};
@@ -138,8 +144,7 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
       f32x16_t x;
 #pragma unroll
       for (int r = 0; r < 16; r++) x[r] = s[0][r] * c_scale_log2;
-      if (CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
-        const int lim = qi - k0 - 4 * h;
+      if (masked) {
 #pragma unroll
         for (int r = 0; r < 16; r++) x[r] = (8 * (r / 4) + (r % 4) <= lim) ? x[r] : -INFINITY;
       }
@@ -172,6 +177,7 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   }
   l += __shfl_xor(l, 32);
   const float inv = 1.f / l;
+  if (qi >= p.n_q) return;
   __bf16* o = (__bf16*)p.o + qoff + (int64_t)qi * p.stride_qn;
 #pragma unroll
   for (int cb = 0; cb < NC; cb++)
@@ -191,18 +197,19 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
-  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[2] = {(const __bf16*)p.k + koff, (const __bf16*)p.v + koff};
 
   bf16x8_t Qb[KK], dOb[KK];
-  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
-  load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
-  const int64_t row = (int64_t)bh * p.n_q + qi;
+  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
+  load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qr, h);
+  const int64_t row = (int64_t)bh * p.n_q + qr;
   const float l_log2 = p.lse[row] * kLog2e, dsum = p.ws_d[row];
   wait_vm0();
   const float c_scale_log2 = p.scale * kLog2e;
@@ -219,12 +226,13 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
 #pragma unroll
   for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
 
-  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  const int k_tiles = (p.n_k + TS - 1) / TS;
+  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
 #pragma unroll
-  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave);
+  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
   dma_wait();
   __syncthreads();
 
@@ -233,9 +241,13 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
 #pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
+    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key);
+    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
+    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
+    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
     if (!CAUSAL || k0 <= qw) {
       const char* stage = smem + (j & 1) * STAGE;
       f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
@@ -246,8 +258,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
       f32x16_t ds;
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * (dp[0][r] - dsum);
-      if (CAUSAL && k0 == qw) {
-        const int lim = qi - k0 - 4 * h;
+      if (masked) {
 #pragma unroll
         for (int r = 0; r < 16; r++) ds[r] = (8 * (r / 4) + (r % 4) <= lim) ? ds[r] : 0.f;
       }
@@ -258,6 +269,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
     dma_wait();
     __syncthreads();
   }
+  if (qi >= p.n_q) return;
   __bf16* o = (__bf16*)p.dq + qoff + (int64_t)qi * p.stride_qn;
 #pragma unroll
   for (int cb = 0; cb < NC; cb++)
@@ -278,18 +290,19 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   constexpr int STAGE = 2 * TILE + STAT;   // Q tile, dO tile, statistics
 
   int bh, tile;
-  if (!decode_block(p.n_k / WG_ROWS, p.batch, false, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int k0 = tile * WG_ROWS, kw = k0 + 32 * wave, kj = kw + n;
+  const int kr = min(kj, p.n_k - 1);  // keys past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[2] = {(const __bf16*)p.q + qoff, (const __bf16*)p.dO + qoff};
-  const float* stat_src = (tid < TS ? p.lse : p.ws_d) + (int64_t)bh * p.n_q + (tid & (TS - 1));
+  const float* stat_src = (tid < TS ? p.lse : p.ws_d) + (int64_t)bh * p.n_q;
 
   bf16x8_t Kb[KK], Vb[KK];
-  load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kj, h);
-  load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kj, h);
+  load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kr, h);
+  load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kr, h);
   const float c_scale_log2 = p.scale * kLog2e;
 
   int aoff[KK], troff[NC][2];
@@ -307,7 +320,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
     acc[1][cb] = f32x16_t{0};
   }
   // causal: query tiles before this workgroup's first key see none of its keys
-  const int t_begin = CAUSAL ? k0 / TS : 0, t_end = p.n_q / TS;
+  const int t_begin = CAUSAL ? k0 / TS : 0, t_end = (p.n_q + TS - 1) / TS;
   Dma<D> dma;
   dma.init(p.stride_qn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
@@ -315,7 +328,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   // The statistic is loaded before the staging loads of a step and first touched at the end of the step, so the
   // wave never waits for it in between.
   auto load_stat = [&](int q_base) {
-    if (tid < 2 * TS) stat_reg = *(global_f32_ptr)(stat_src + q_base);
+    if (tid < 2 * TS) stat_reg = *(global_f32_ptr)(stat_src + min(q_base + (tid & (TS - 1)), p.n_q - 1));
   };
   auto store_stat = [&](char* stage_base) {
     if (tid < 2 * TS) reinterpret_cast<float*>(stage_base + 2 * TILE)[tid] = (tid < TS) ? stat_reg * kLog2e : stat_reg;
@@ -324,7 +337,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
     load_stat(t_begin * TS);
     const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
 #pragma unroll
-    for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x] + adv, wave);
+    for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x] + adv, wave, p.n_q - t_begin * TS);
     wait_vm0();
     store_stat(smem);
   }
@@ -337,7 +350,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
       const uint32_t dst = ring_lds + (st ^ 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
 #pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_q - (j + 1) * TS);
     }
     const int qb = j * TS;
     if (!CAUSAL || qb >= kw) {  // else no query of the tile sees a key of this wave
@@ -360,10 +373,14 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
           ds[r] = dp[0][r] - d4[e];
         }
       }
-      if (CAUSAL && qb == kw) {  // wave-uniform: only the block on the diagonal
-        const int lim = kj - qb - 4 * h;  // query row 8g + 4h + e sees key kj iff 8g + e >= lim
+      if ((CAUSAL && qb == kw) || qb + TS > p.n_q) {  // wave-uniform: diagonal block, or the block with the last query
+        // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it sees key kj and exists
+        const int lo = (CAUSAL && qb == kw ? kj - qb : 0) - 4 * h, hi = p.n_q - 1 - qb - 4 * h;
 #pragma unroll
-        for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) >= lim) ? pv[r] : 0.f;
+        for (int r = 0; r < 16; r++) {
+          const int x = 8 * (r / 4) + (r % 4);
+          pv[r] = (x >= lo && x <= hi) ? pv[r] : 0.f;
+        }
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] *= pv[r];
@@ -378,6 +395,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
     dma_wait();
     __syncthreads();
   }
+  if (kj >= p.n_k) return;
   __bf16* odk = (__bf16*)p.dk + koff + (int64_t)kj * p.stride_kn;
   __bf16* odv = (__bf16*)p.dv + koff + (int64_t)kj * p.stride_kn;
 #pragma unroll
@@ -404,9 +422,9 @@ template <bool F16, int D, bool CAUSAL>
 hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
   constexpr int TILE = TS * 2 * D;
   switch (which) {
-    case 0: return launch(attn_fwd_bf16<F16, D, CAUSAL>, grid_blocks(p.n_q / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    case 1: return launch(attn_bwd_q_bf16<F16, D, CAUSAL>, grid_blocks(p.n_q / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    default: return launch(attn_bwd_k_bf16<F16, D, CAUSAL>, grid_blocks(p.n_k / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
+    case 0: return launch(attn_fwd_bf16<F16, D, CAUSAL>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    case 1: return launch(attn_bwd_q_bf16<F16, D, CAUSAL>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    default: return launch(attn_bwd_k_bf16<F16, D, CAUSAL>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
   }
 }
 

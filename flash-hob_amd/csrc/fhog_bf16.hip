@@ -31,21 +31,22 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   constexpr int KK = D / 16;
 
   int bh, tile;
-  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
                           (const __bf16*)p.ddv + koff};
 
   bf16x8_t Qb[KK], ddQb[KK], dOb[KK];
-  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
-  load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qi, h);
-  if (PASS != 1) load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
+  load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
+  load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qr, h);
+  if (PASS != 1) load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qr, h);
 
-  const int64_t row = (int64_t)bh * p.n_q + qi;
+  const int64_t row = (int64_t)bh * p.n_q + qr;
   const float l_log2 = p.lse[row] * kLog2e;
   const float c_scale_log2 = p.scale * kLog2e;
   const float dsum = PASS != 1 ? p.ws_d[row] : 0.f;
@@ -60,12 +61,13 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
 
-  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  const int k_tiles = (p.n_k + TS - 1) / TS;
+  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
 #pragma unroll
-  for (int x = 0; x < NT; x++) dma.issue(ring_lds + x * TILE, src[x], wave);
+  for (int x = 0; x < NT; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
   dma_wait();
   __syncthreads();
 
@@ -74,9 +76,13 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
 #pragma unroll
-      for (int x = 0; x < NT; x++) dma.issue(dst + x * TILE, src[x] + adv, wave);
+      for (int x = 0; x < NT; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
+    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key)
+    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
+    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
+    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
     if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
       const char* stage = smem + (j & 1) * STAGE;
       // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
@@ -120,8 +126,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
           }
         } else {
           e = mfma<F16>(a[c], dOb[kk], e);
-          if (kk == 0 && CAUSAL && k0 == qw) {  // wave-uniform: only the block on the diagonal
-            const int lim = qi - k0 - 4 * h;
+          if (kk == 0 && masked) {
 #pragma unroll
             for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
           }
@@ -139,8 +144,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
         __builtin_amdgcn_sched_barrier(0);
       }
       if (PASS == 1) {
-        if (CAUSAL && k0 == qw) {
-          const int lim = qi - k0 - 4 * h;
+        if (masked) {
 #pragma unroll
           for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
         }
@@ -163,11 +167,11 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
     red_dd += __shfl_xor(red_dd, 32);
     red_pdp += __shfl_xor(red_pdp, 32);
     const float dd_i = red_dd * p.scale;
-    if (h == 0) {
+    if (h == 0 && qi < p.n_q) {
       p.ws_dd[row] = dd_i;
       p.ws_b[row] = __builtin_fmaf(-dd_i, red_pdp, red);
     }
-  } else if (h == 0) {
+  } else if (h == 0 && qi < p.n_q) {
     (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
   }
 }
@@ -175,7 +179,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
 template <bool F16, int D, bool CAUSAL>
 hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(256);
-  const dim3 grid(grid_blocks(p.n_q / WG_ROWS, p.batch));
+  const dim3 grid(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch));
   const int tile = TS * 2 * D;
   hipError_t e;
   if (pass == FHOG_PASS_DD) {
@@ -203,7 +207,7 @@ hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s);
 
 bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
   (void)causal;
-  return (d == 64 || d == 128) && n_q % WG_ROWS == 0 && n_k % WG_ROWS == 0;
+  return (d == 64 || d == 128) && n_q >= 1 && n_k >= 1;
 }
 
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {

@@ -63,7 +63,7 @@ __device__ __forceinline__ void sop_write_group(char* tile, uint32_t lo, uint32_
 
 template <bool F16, int D>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
-                                          const bf16x8_t* dOb, int lane, int q_idx, int k_base, bool mask,
+                                          const bf16x8_t* dOb, int lane, int lim, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
   constexpr int TILE = TS * 2 * D;
   constexpr int KK = D / 16, NSTEP = 4 * KK, PF = 2, NB = PF + 1;
@@ -95,8 +95,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
     } else if (ph == 2) {
       dds = mfma<F16>(a[c], Qb[kk], dds);
-      if (kk == 0 && mask) {  // wave-uniform: only the block on the diagonal
-        const int lim = q_idx - k_base - 4 * h;
+      if (kk == 0 && mask) {  // wave-uniform: the block lies on the diagonal or reaches past the last key
 #pragma unroll
         for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
       }
@@ -149,7 +148,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   constexpr int NC = D / 32;
 
   int bh, tile;
-  if (!decode_block(p.n_q / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
@@ -157,15 +156,17 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wq, qi = qw + n;
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
-  const int n_tiles = CAUSAL ? (q0 + WG_ROWS) / TS : p.n_k / TS;
+  const int k_tiles = (p.n_k + TS - 1) / TS;
+  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
     bf16x8_t Qb[D / 16], ddQb[D / 16], dOb[D / 16];
-    load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qi, h);
-    load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qi, h);
-    load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qi, h);
-    const int64_t row = (int64_t)bh * p.n_q + qi;
+    const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row; nothing of them is stored
+    load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
+    load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qr, h);
+    load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qr, h);
+    const int64_t row = (int64_t)bh * p.n_q + qr;
     const float l_log2 = p.lse[row] * kLog2e;
     const float c_scale_log2 = p.scale * kLog2e;
     const float dsum = p.ws_d[row], dd = p.ws_dd[row], b = p.ws_b[row];
@@ -176,7 +177,10 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       if (j < n_tiles && (!CAUSAL || k0 <= qw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, qi, k0, CAUSAL && k0 == qw, c_scale_log2, l_log2, p.scale, dsum, dd, b);
+        // key k0 + 8g + 4h + e is visible iff 8g + e <= lim (diagonal block, or the block that holds the last key)
+        const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
+        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, lim, (CAUSAL && k0 == qw) || k0 + TS > p.n_k, c_scale_log2, l_log2,
+                          p.scale, dsum, dd, b);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -208,7 +212,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
     dma.init(p.stride_kn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
 #pragma unroll
-    for (int x = 0; x < 4; x++) dma.issue(ring_lds + x * SM::TILE, src[x], wq);
+    for (int x = 0; x < 4; x++) dma.issue(ring_lds + x * SM::TILE, src[x], wq, p.n_k);
     dma_wait();
     __syncthreads();
     int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
@@ -217,7 +221,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
         const uint32_t dst = ring_lds + sn * SM::STAGE;
         const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
 #pragma unroll
-        for (int x = 0; x < 4; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
+        for (int x = 0; x < 4; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq, p.n_k - (j + 1) * TS);
       }
       // block j-1: query block qb of the pair took part iff its first query is not before the tile
       const bool act0 = j >= 1 && (!CAUSAL || (j - 1) * TS <= qw0);
@@ -285,9 +289,12 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       for (int cl = 0; cl < NCL; cl++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const int64_t o = (int64_t)(qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_qn + 32 * (NCL * ch + cl) + n;
-          odq[o] = to_elem<F16>(acc_dq[qb][cl][r] * p.scale);
-          oddo[o] = to_elem<F16>(acc_ddo[qb][cl][r]);
+          const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
+          if (qrow < p.n_q) {
+            const int64_t o = (int64_t)qrow * p.stride_qn + 32 * (NCL * ch + cl) + n;
+            odq[o] = to_elem<F16>(acc_dq[qb][cl][r] * p.scale);
+            oddo[o] = to_elem<F16>(acc_ddo[qb][cl][r]);
+          }
         }
   }
 }
@@ -295,7 +302,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 // ---- pass 4 ------------------------------------------------------------------------------------------
 template <bool F16, int D>
 __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* ddKb,
-                                          const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int k_idx, int q_base,
+                                          const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int lo, int hi,
                                           bool mask, float c_scale_log2, float scale) {
   constexpr int TILE = TS * 2 * D;
   const int n = lane & 31, h = lane >> 5;
@@ -335,10 +342,12 @@ __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf
 #pragma unroll
     for (int j = 0; j < 4; j++) pv[4 * g + j] = __builtin_amdgcn_exp2f(s[4 * g + j] * c_scale_log2 - l4[j]);
   }
-  if (mask) {  // wave-uniform: only the block on the diagonal
-    const int lim = k_idx - q_base - 4 * h;   // query row 8g + 4h + j sees key k_idx iff 8g + j >= lim
+  if (mask) {  // wave-uniform: the block lies on the diagonal or reaches past the last query
 #pragma unroll
-    for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) >= lim) ? pv[r] : 0.f;
+    for (int r = 0; r < 16; r++) {
+      const int x = 8 * (r / 4) + (r % 4);  // query row 8g + 4h + j of the tile counts iff lo <= 8g + j <= hi
+      pv[r] = (x >= lo && x <= hi) ? pv[r] : 0.f;
+    }
   }
 #pragma unroll
   for (int g = 0; g < 4; g++) {
@@ -369,25 +378,26 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   constexpr int NC = D / 32;
 
   int bh, tile;
-  if (!decode_block(p.n_k / WG_ROWS, p.batch, false, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
   const int wq = wave & 3;
   const int n = lane & 31, h = lane >> 5;
   const int k0 = tile * WG_ROWS, kw = k0 + 32 * wq, kj = kw + n;
+  const int kr = min(kj, p.n_k - 1);  // keys past the end compute on a copy of the last row; nothing of them is stored
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   // causal: query tiles before this workgroup's first key see none of its keys
   const int t_begin = CAUSAL ? k0 / TS : 0;
-  const int t_end = p.n_q / TS;
+  const int t_end = (p.n_q + TS - 1) / TS;
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
     bf16x8_t Kb[D / 16], ddKb[D / 16], Vb[D / 16], ddVb[D / 16];
-    load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kj, h);
-    load_resident<D>(ddKb, (const __bf16*)p.ddk + koff, p.stride_kn, kj, h);
-    load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kj, h);
-    load_resident<D>(ddVb, (const __bf16*)p.ddv + koff, p.stride_kn, kj, h);
+    load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kr, h);
+    load_resident<D>(ddKb, (const __bf16*)p.ddk + koff, p.stride_kn, kr, h);
+    load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kr, h);
+    load_resident<D>(ddVb, (const __bf16*)p.ddv + koff, p.stride_kn, kr, h);
     const float c_scale_log2 = p.scale * kLog2e;
     __syncthreads();
     int sp = 0;  // ring slot of tile j (slot 0 holds tile t_begin)
@@ -396,7 +406,10 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       if (j < t_end && (!CAUSAL || qb >= kw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, kj, qb, CAUSAL && qb == kw, c_scale_log2, p.scale);
+        // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it sees key kj (diagonal block) and exists
+        const int lo = (CAUSAL && qb == kw ? kj - qb : 0) - 4 * h, hi = p.n_q - 1 - qb - 4 * h;
+        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, lo, hi, (CAUSAL && qb == kw) || qb + TS > p.n_q, c_scale_log2,
+                          p.scale);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -427,7 +440,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     // The loaded value is first touched in store_stat, at the end of the step: a use right after the load would
     // make the wave wait there for the load and, with it, for every staging load issued before it.
     auto load_stat = [&](int q_base) {
-      if (ctid < 4 * TS) stat_reg = *(global_f32_ptr)(stat_src[ctid / TS] + q_base + (ctid % TS));
+      if (ctid < 4 * TS) stat_reg = *(global_f32_ptr)(stat_src[ctid / TS] + min(q_base + (ctid % TS), p.n_q - 1));
     };
     auto store_stat = [&](char* stage_base) {
       if (ctid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * SM::TILE)[ctid] = (ctid < TS) ? stat_reg * kLog2e : stat_reg;
@@ -435,7 +448,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     {
       const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
 #pragma unroll
-      for (int x = 0; x < 3; x++) dma.issue(ring_lds + x * SM::TILE, src[x] + adv, wq);
+      for (int x = 0; x < 3; x++) dma.issue(ring_lds + x * SM::TILE, src[x] + adv, wq, p.n_q - t_begin * TS);
       load_stat(t_begin * TS);
       store_stat(smem);
     }
@@ -448,7 +461,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
         const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
         load_stat((j + 1) * TS);
 #pragma unroll
-        for (int x = 0; x < 3; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq);
+        for (int x = 0; x < 3; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq, p.n_q - (j + 1) * TS);
       }
       if (j > t_begin && (!CAUSAL || (j - 1) * TS >= kw)) {
         const char* stage = smem + sc * SM::STAGE;
@@ -496,9 +509,12 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     for (int cb = 0; cb < NC; cb++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int64_t o = (int64_t)(kw + 8 * (r / 4) + 4 * h + (r % 4)) * p.stride_kn + cb * 32 + n;
-        odk[o] = to_elem<F16>(acc_dk[cb][r] * p.scale);
-        odv[o] = to_elem<F16>(acc_dv[cb][r]);
+        const int krow = kw + 8 * (r / 4) + 4 * h + (r % 4);
+        if (krow < p.n_k) {
+          const int64_t o = (int64_t)krow * p.stride_kn + cb * 32 + n;
+          odk[o] = to_elem<F16>(acc_dk[cb][r] * p.scale);
+          odv[o] = to_elem<F16>(acc_dv[cb][r]);
+        }
       }
   }
 }
@@ -511,12 +527,12 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
     const int smem = PCSmem<D, false>::TOTAL;
     e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep3_pc<F16, D, CAUSAL>), dim3(grid_blocks(p.n_q / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep3_pc<F16, D, CAUSAL>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
   } else {
     const int smem = PCSmem<D, true>::TOTAL;
     e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_sweep_pc<F16, D, CAUSAL>), dim3(grid_blocks(p.n_k / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((k_sweep_pc<F16, D, CAUSAL>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
   }
   return hipGetLastError();
 }

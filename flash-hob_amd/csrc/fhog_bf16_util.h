@@ -113,21 +113,31 @@ struct Dma {
   static constexpr int IPT = TS / RPI;          // instructions per 32-row tile (8 or 4)
   static constexpr int PER_WAVE = IPT / 4;      // instructions per tile for each of 4 loader waves (2 or 1)
   uint32_t voff[PER_WAVE];                      // per-lane byte offset from the tile's first row
+  int64_t ld_;
+  int lw_, lane_;
 
-  __device__ __forceinline__ void init(int64_t ld, int lw, int lane) {
-#pragma unroll
-    for (int u = 0; u < PER_WAVE; u++) {
-      const int q = lw + 4 * u;
-      const int r = q * RPI + lane / CPR, pc = lane % CPR;
-      voff[u] = (uint32_t)((r * ld + ((pc ^ swz<D>(r)) << 3)) * 2);
-    }
+  __device__ __forceinline__ uint32_t lane_offset(int u, int rows_valid) const {
+    const int q = lw_ + 4 * u;
+    const int r = q * RPI + lane_ / CPR, pc = lane_ % CPR;
+    const int rs = r < rows_valid ? r : rows_valid - 1;  // rows past the end of the tensor re-read its last row
+    return (uint32_t)((rs * ld_ + ((pc ^ swz<D>(r)) << 3)) * 2);
   }
-  // tile_lds: LDS byte address of the destination tile (wave-uniform); src: first row of the source tile
-  __device__ __forceinline__ void issue(uint32_t tile_lds, const __bf16* src, int lw) const {
+  __device__ __forceinline__ void init(int64_t ld, int lw, int lane) {
+    ld_ = ld;
+    lw_ = lw;
+    lane_ = lane;
+#pragma unroll
+    for (int u = 0; u < PER_WAVE; u++) voff[u] = lane_offset(u, TS);
+  }
+  // tile_lds: LDS byte address of the destination tile (wave-uniform); src: first row of the source tile;
+  // rows_valid: rows of the tensor from that row on (>= TS for a full tile). A partial tile is filled up with copies of
+  // the tensor's last row, so that no load leaves the tensor; the kernels mask those rows.
+  __device__ __forceinline__ void issue(uint32_t tile_lds, const __bf16* src, int lw, int rows_valid = TS) const {
 #pragma unroll
     for (int u = 0; u < PER_WAVE; u++) {
       const uint32_t m0 = __builtin_amdgcn_readfirstlane(tile_lds + (lw + 4 * u) * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(voff[u]), "s"(src) : "memory", "m0");
+      const uint32_t off = rows_valid >= TS ? voff[u] : lane_offset(u, rows_valid);
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
     }
   }
 };

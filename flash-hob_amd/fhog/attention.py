@@ -11,7 +11,7 @@ commented stub (``fhog/triton_bwdbwd.py:538-554``).  Here it is wired:
     AttnBwd.backward         -> flash_bwdbwd(...) -> dQ', dK', dV', ddO
 
 The forward and the first-order backward are the callers on either side of the hot path.  For bf16 and fp16
-tensors with d in {64, 128} and sequence lengths that are multiples of 128 they run as HIP kernels of
+tensors with d in {64, 128} they run as HIP kernels of
 the same library (``fhog_attn_fwd`` / ``fhog_attn_bwd``); every other dtype or shape takes
 linear-memory torch compositions on the GPU (blocked over heads and query rows, fp32 accumulation).
 The double-backward is always the HIP library.
@@ -149,7 +149,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, w
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16/fp16, d in {64,128}, N multiple of 128, GPU)")
+            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16/fp16, d in {64,128}, GPU)")
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
@@ -178,7 +178,7 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal, *, window: Optio
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16/fp16, d in {64,128}, N multiple of 128, GPU)")
+            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16/fp16, d in {64,128}, GPU)")
     dq = torch.empty_like(q)
     dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)

@@ -136,7 +136,7 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream);
 
 /* ---- first-order attention: the callers on either side of the double-backward ---------------------------
- * bf16 or fp16 tensors, d in {64, 128}, n_q and n_k multiples of 128 (fhog_attn_supported tells); the layout rules
+ * bf16 or fp16 tensors, d in {64, 128}, any n_q and n_k (fhog_attn_validate tells); the layout rules
  * above apply. O and dO/dQ share the q strides, dK/dV the k strides. */
 typedef struct fhog_attn_args {
   const void* q;   /* (batch, n_q, d) */

@@ -79,7 +79,7 @@ def good_attn_args():
     (lambda a: setattr(a, "dO", 0), 1, -1, "dO"),
     (lambda a: setattr(a, "lse", 0), 0, -1, "lse"),
     (lambda a: setattr(a, "dtype", 1), 0, -3, "bf16"),
-    (lambda a: setattr(a, "n_q", 200), 0, -2, "multiples of 128"),
+    (lambda a: setattr(a, "n_q", 200), 0, 0, ""),           # ragged lengths are fine
     (lambda a: setattr(a, "d", 32), 0, -2, "d in"),
     (lambda a: setattr(a, "causal", 1), 0, -6, "causal"),
     (lambda a: setattr(a, "stride_kn", 60), 0, -4, "stride"),
@@ -173,8 +173,11 @@ def test_impl_bf16_needs_bf16_shape(L):
     a.dtype = 1
     assert L.fhog_validate(ctypes.byref(a)) == -3
     a.dtype = 0
-    a.n_q = 100
+    a.n_q = 100                      # ragged lengths are taken by the 16-bit kernels
     a.stride_qb = 100 * 64
+    assert L.fhog_validate(ctypes.byref(a)) == 0
+    a.d = 32                         # d = 32 is not
+    a.stride_qn = a.stride_kn = 32
     assert L.fhog_validate(ctypes.byref(a)) == -2
 
 

@@ -234,6 +234,43 @@ def test_single_head_spreads_over_the_chip():
     assert max(e.values()) < 2e-2, e
 
 
+@pytest.mark.parametrize("fused_stats", [False, True])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(3, 100, 77, 64), (2, 33, 129, 128), (2, 333, 333, 128), (1, 1, 1, 64), (2, 31, 31, 128),
+                                   (2, 129, 257, 64), (1, 1000, 1000, 128), (5, 160, 96, 64)])
+def test_bf16_family_ragged_lengths(shape, causal, fused_stats):
+    """Sequence lengths that are no multiple of the 128-row workgroup tile or of the 32-row stage: rows past the end
+    are computed on copies of the last row and masked / not stored."""
+    batch, n_q, n_k, d = shape
+    if causal:
+        n_k = n_q
+    x = make_case(batch, n_q, n_k, d, torch.bfloat16, seed=18, grad_std=0.1)
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal)
+    canary = 7.0
+    outs = run_fhog(x, scale, causal, impl="bf16", return_stats=True, fused_stats=fused_stats)
+    ref = reference_fp64_cpu(x, scale, causal)
+    e = errors(outs[:4], [ref[n] for n in NAMES])
+    assert max(e.values()) < 2e-2, e
+    for got, name in zip(outs[4], ("d", "dd", "b")):
+        assert normalised_max_error(got, ref[name]) < 1e-2, name
+    # nothing is written past the end of a tensor: outputs are views into larger canary-filled buffers
+    from fhog import BwdBwdPlan
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], scale, causal=causal,
+                      impl="bf16", fused_stats=fused_stats)
+    big = [torch.full((t.numel() + 4096,), canary, dtype=t.dtype, device=t.device) for t in plan.outs]
+    ws_big = torch.full((plan.ws.numel() + 1024,), canary, dtype=torch.float32, device="cuda")
+    for name, buf, t in zip(("dq2", "dk2", "dv2", "ddo"), big, plan.outs):
+        setattr(plan.args, name, buf.data_ptr())
+    plan.args.ws = ws_big.data_ptr()
+    plan.run()
+    torch.cuda.synchronize()
+    for buf, t, o in zip(big, plan.outs, outs[:4]):
+        assert torch.equal(buf[:t.numel()].view(t.shape), o.reshape(t.shape))
+        assert (buf[t.numel():] == canary).all()
+    assert (ws_big[plan.ws.numel():] == canary).all()
+
+
 def test_bf16_auto_dispatch():
     from fhog import BwdBwdPlan
     x = with_caches(make_case(2, 256, 256, 64, torch.bfloat16, seed=6), 0.125, False)
@@ -241,7 +278,10 @@ def test_bf16_auto_dispatch():
     assert plan.impl == 2
     y = with_caches(make_case(2, 200, 256, 64, torch.bfloat16, seed=6), 0.125, False)
     plan = BwdBwdPlan(y["Q"], y["K"], y["V"], y["O"], y["dO"], y["ddQ"], y["ddK"], y["ddV"], y["L"], 0.125)
-    assert plan.impl == 1
+    assert plan.impl == 2          # ragged lengths stay on the 16-bit kernels
+    z = with_caches(make_case(2, 128, 128, 32, torch.bfloat16, seed=6), 32 ** -0.5, False)
+    plan = BwdBwdPlan(z["Q"], z["K"], z["V"], z["O"], z["dO"], z["ddQ"], z["ddK"], z["ddV"], z["L"], 32 ** -0.5)
+    assert plan.impl == 1          # d = 32 is served by the fp32-MFMA kernels
 
 
 def _full_config(name, seed, heads=None, fused_stats=False):
