@@ -21,10 +21,22 @@ int fail(int code, const char* fmt, ...) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// no mask, or the square causal mask with no effective window: what the 16-bit kernels implement
-bool plain_mask(const fhog_bwdbwd_args* a) {
-  if (a->causal == FHOG_MASK_NONE) return true;
-  return a->n_q == a->n_k && (a->window == 0 || a->window >= a->n_k);
+// FHOG_OK or the error for a mask that does not apply to the shape
+int check_mask(int32_t causal, int64_t window, int64_t n_q, int64_t n_k) {
+  if (causal < FHOG_MASK_NONE || causal > FHOG_MASK_BOTTOM_RIGHT) return fail(FHOG_E_CAUSAL, "causal must be 0, 1 or 2");
+  if (causal == FHOG_MASK_TOP_LEFT && n_q != n_k)
+    return fail(FHOG_E_CAUSAL, "causal (top-left) needs n_q == n_k (got %lld, %lld)", (long long)n_q, (long long)n_k);
+  if (causal == FHOG_MASK_BOTTOM_RIGHT && n_k < n_q)
+    return fail(FHOG_E_CAUSAL, "causal (bottom-right) needs n_k >= n_q (got %lld, %lld)", (long long)n_k, (long long)n_q);
+  if (window < 0) return fail(FHOG_E_CAUSAL, "window must be >= 0");
+  if (window > 0 && causal == FHOG_MASK_NONE) return fail(FHOG_E_CAUSAL, "a window needs a causal mask");
+  return FHOG_OK;
+}
+// kernel-side mask parameters: key j is visible to query i iff 0 <= i + off - j < win
+void mask_params(int32_t causal, int64_t window, int64_t n_q, int64_t n_k, int32_t* off, int32_t* win) {
+  *off = causal == FHOG_MASK_BOTTOM_RIGHT ? (int32_t)(n_k - n_q) : 0;
+  const int64_t reach = n_q + n_k;  // a window this long hides nothing
+  *win = (int32_t)((window == 0 || window > reach) ? reach : window);
 }
 
 int validate(const fhog_bwdbwd_args* a) {
@@ -46,13 +58,7 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->n_q > (1 << 24) || a->n_k > (1 << 24)) return fail(FHOG_E_SHAPE, "n_q/n_k above 2^24 not supported");
   if (a->batch * a->n_q >= (int64_t)1 << 31) return fail(FHOG_E_SHAPE, "batch*n_q must be below 2^31");
   if (a->d != 32 && a->d != 64 && a->d != 128) return fail(FHOG_E_SHAPE, "head dim %lld not in {32, 64, 128}", (long long)a->d);
-  if (a->causal < FHOG_MASK_NONE || a->causal > FHOG_MASK_BOTTOM_RIGHT) return fail(FHOG_E_CAUSAL, "causal must be 0, 1 or 2");
-  if (a->causal == FHOG_MASK_TOP_LEFT && a->n_q != a->n_k)
-    return fail(FHOG_E_CAUSAL, "causal (top-left) needs n_q == n_k (got %lld, %lld)", (long long)a->n_q, (long long)a->n_k);
-  if (a->causal == FHOG_MASK_BOTTOM_RIGHT && a->n_k < a->n_q)
-    return fail(FHOG_E_CAUSAL, "causal (bottom-right) needs n_k >= n_q (got %lld, %lld)", (long long)a->n_k, (long long)a->n_q);
-  if (a->window < 0) return fail(FHOG_E_CAUSAL, "window must be >= 0");
-  if (a->window > 0 && a->causal == FHOG_MASK_NONE) return fail(FHOG_E_CAUSAL, "a window needs a causal mask");
+  if (const int rc = check_mask(a->causal, a->window, a->n_q, a->n_k)) return rc;
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
   const int vec = a->dtype == FHOG_DTYPE_FP32 ? 4 : 8;  // elements per 16 bytes
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
@@ -66,7 +72,6 @@ int validate(const fhog_bwdbwd_args* a) {
     if (a->dtype == FHOG_DTYPE_FP32) return fail(FHOG_E_DTYPE, "impl=bf16 needs bf16 or fp16 tensors");
     if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
       return fail(FHOG_E_SHAPE, "impl=bf16 needs d in {64,128}");
-    if (!plain_mask(a)) return fail(FHOG_E_CAUSAL, "impl=bf16 takes no mask or the square causal mask without a window");
   }
   return FHOG_OK;
 }
@@ -74,8 +79,7 @@ int validate(const fhog_bwdbwd_args* a) {
 int select_impl(const fhog_bwdbwd_args* a) {
   if (a->impl == FHOG_IMPL_FP32) return FHOG_IMPL_FP32;
   if (a->impl == FHOG_IMPL_BF16) return FHOG_IMPL_BF16;
-  if (a->dtype != FHOG_DTYPE_FP32 && plain_mask(a) && fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
-    return FHOG_IMPL_BF16;
+  if (a->dtype != FHOG_DTYPE_FP32 && fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal)) return FHOG_IMPL_BF16;
   return FHOG_IMPL_FP32;
 }
 
@@ -109,9 +113,7 @@ fhog::Params to_params(const fhog_bwdbwd_args* a) {
   p.scale = a->scale;
   p.causal = a->causal != FHOG_MASK_NONE;
   p.f16 = a->dtype == FHOG_DTYPE_FP16;
-  p.mask_off = a->causal == FHOG_MASK_BOTTOM_RIGHT ? (int32_t)(a->n_k - a->n_q) : 0;
-  const int64_t reach = a->n_q + a->n_k;  // a window this long masks nothing
-  p.window = (int32_t)((a->window == 0 || a->window > reach) ? reach : a->window);
+  mask_params(a->causal, a->window, a->n_q, a->n_k, &p.mask_off, &p.window);
   return p;
 }
 
@@ -144,8 +146,7 @@ int validate_attn(const fhog_attn_args* a, int backward) {
   if (a->batch < 1 || a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld outside 1..65535", (long long)a->batch);
   if (a->n_q < 1 || a->n_k < 1 || a->n_q > (1 << 24) || a->n_k > (1 << 24) || a->batch * a->n_q >= (int64_t)1 << 31)
     return fail(FHOG_E_SHAPE, "n_q/n_k out of range");
-  if (a->causal != 0 && a->causal != 1) return fail(FHOG_E_CAUSAL, "causal must be 0 or 1");
-  if (a->causal && a->n_q != a->n_k) return fail(FHOG_E_CAUSAL, "causal needs n_q == n_k");
+  if (const int rc = check_mask(a->causal, a->window, a->n_q, a->n_k)) return rc;
   if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
     return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128}");
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
@@ -178,8 +179,9 @@ fhog::AttnParams to_attn_params(const fhog_attn_args* a) {
   p.n_k = (int32_t)a->n_k;
   p.d = (int32_t)a->d;
   p.scale = a->scale;
-  p.causal = a->causal;
+  p.causal = a->causal != FHOG_MASK_NONE;
   p.f16 = a->dtype == FHOG_DTYPE_FP16;
+  mask_params(a->causal, a->window, a->n_q, a->n_k, &p.mask_off, &p.window);
   return p;
 }
 

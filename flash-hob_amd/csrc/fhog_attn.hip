@@ -81,13 +81,13 @@ __device__ __forceinline__ void first_level(const char* tile, const int (&aoff)[
 }
 
 // ---- forward -----------------------------------------------------------------------------------------
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -114,29 +114,27 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
 #pragma unroll
   for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
 
-  const int k_tiles = (p.n_k + TS - 1) / TS;
-  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;  // key tiles this workgroup visits
+  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-#pragma unroll
-  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
+  dma.template issue_all<2>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
-  for (int j = 0; j < n_tiles; j++) {
-    if (j + 1 < n_tiles) {
+  for (int j = j_begin; j < j_end; j++) {
+    if (j + 1 < j_end) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-#pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
+      dma.template issue_all<2>(dst, TILE, src, adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
-    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key);
-    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
-    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
-    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
-    if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
+    const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
+    int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
+    if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
+    if (!geo.dead(k0, qw)) {  // else every key of the tile is hidden from this wave
       const char* stage = smem + (j & 1) * STAGE;
       f32x16_t s[1] = {f32x16_t{0}};
       const bf16x8_t* const res[1] = {Qb};
@@ -145,19 +143,22 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) x[r] = s[0][r] * c_scale_log2;
       if (masked) {
+        keep_branch();
 #pragma unroll
-        for (int r = 0; r < 16; r++) x[r] = (8 * (r / 4) + (r % 4) <= lim) ? x[r] : -INFINITY;
+        for (int r = 0; r < 16; r++) x[r] = in_limits(r, lo, hi) ? x[r] : -INFINITY;
       }
       float tmax = x[0];
 #pragma unroll
       for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, x[r]);
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-      const float m_new = fmaxf(m, tmax);  // finite: key 0 is visible to every query and tiles come in key order
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      const float m_new = fmaxf(m, tmax);
+      // a row whose window starts in a later tile has seen no key yet: keep exp2(-inf - (-inf)) out of it
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
       float rs = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        x[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+        x[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
         rs += x[r];
       }
       l = __builtin_fmaf(l, alpha, rs);
@@ -191,13 +192,13 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
 }
 
 // ---- backward, Q-tiled: dQ -----------------------------------------------------------------------------
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -226,29 +227,27 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
 #pragma unroll
   for (int cb = 0; cb < NC; cb++) acc[0][cb] = f32x16_t{0};
 
-  const int k_tiles = (p.n_k + TS - 1) / TS;
-  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;  // key tiles this workgroup visits
+  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-#pragma unroll
-  for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
+  dma.template issue_all<2>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
-  for (int j = 0; j < n_tiles; j++) {
-    if (j + 1 < n_tiles) {
+  for (int j = j_begin; j < j_end; j++) {
+    if (j + 1 < j_end) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-#pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
+      dma.template issue_all<2>(dst, TILE, src, adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
-    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key);
-    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
-    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
-    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
-    if (!CAUSAL || k0 <= qw) {
+    const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
+    int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
+    if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
+    if (!geo.dead(k0, qw)) {
       const char* stage = smem + (j & 1) * STAGE;
       f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
       const bf16x8_t* const rq[1] = {Qb};
@@ -259,8 +258,9 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * (dp[0][r] - dsum);
       if (masked) {
+        keep_branch();
 #pragma unroll
-        for (int r = 0; r < 16; r++) ds[r] = (8 * (r / 4) + (r % 4) <= lim) ? ds[r] : 0.f;
+        for (int r = 0; r < 16; r++) ds[r] = in_limits(r, lo, hi) ? ds[r] : 0.f;
       }
       const bf16x8_t op[1][2] = {{pack_operand<F16>(ds, 0), pack_operand<F16>(ds, 1)}};
       const char* const kt[1] = {stage};
@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
 }
 
 // ---- backward, K-tiled: dK, dV ---------------------------------------------------------------------------
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
@@ -319,8 +319,9 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
     acc[0][cb] = f32x16_t{0};
     acc[1][cb] = f32x16_t{0};
   }
-  // causal: query tiles before this workgroup's first key see none of its keys
-  const int t_begin = CAUSAL ? k0 / TS : 0, t_end = (p.n_q + TS - 1) / TS;
+  const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
+  int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
+  geo.tile_range(k0, WG_ROWS, t_begin, t_end);
   Dma<D> dma;
   dma.init(p.stride_qn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
@@ -336,8 +337,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   {
     load_stat(t_begin * TS);
     const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
-#pragma unroll
-    for (int x = 0; x < 2; x++) dma.issue(ring_lds + x * TILE, src[x] + adv, wave, p.n_q - t_begin * TS);
+    dma.template issue_all<2>(ring_lds, TILE, src, adv, wave, p.n_q - t_begin * TS);
     wait_vm0();
     store_stat(smem);
   }
@@ -349,11 +349,10 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
       load_stat((j + 1) * TS);
       const uint32_t dst = ring_lds + (st ^ 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
-#pragma unroll
-      for (int x = 0; x < 2; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_q - (j + 1) * TS);
+      dma.template issue_all<2>(dst, TILE, src, adv, wave, p.n_q - (j + 1) * TS);
     }
     const int qb = j * TS;
-    if (!CAUSAL || qb >= kw) {  // else no query of the tile sees a key of this wave
+    if (!geo.dead(qb, kw)) {  // else no query of the tile sees a key of this wave
       const char* stage = smem + st * STAGE;
       const float* stat = reinterpret_cast<const float*>(stage + 2 * TILE);
       f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
@@ -373,14 +372,12 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
           ds[r] = dp[0][r] - d4[e];
         }
       }
-      if ((CAUSAL && qb == kw) || qb + TS > p.n_q) {  // wave-uniform: diagonal block, or the block with the last query
-        // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it sees key kj and exists
-        const int lo = (CAUSAL && qb == kw ? kj - qb : 0) - 4 * h, hi = p.n_q - 1 - qb - 4 * h;
+      if (geo.partial(qb, kw)) {  // wave-uniform: the block holds hidden (query, key) pairs
+        int lo, hi;                // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it exists and sees key kj
+        geo.limits(qb, kj, h, lo, hi);
+        keep_branch();
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int x = 8 * (r / 4) + (r % 4);
-          pv[r] = (x >= lo && x <= hi) ? pv[r] : 0.f;
-        }
+        for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) ds[r] *= pv[r];
@@ -418,13 +415,13 @@ hipError_t launch(K kernel, unsigned grid, int smem, hipStream_t s, const AttnPa
   return hipGetLastError();
 }
 
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
   constexpr int TILE = TS * 2 * D;
   switch (which) {
-    case 0: return launch(attn_fwd_bf16<F16, D, CAUSAL>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    case 1: return launch(attn_bwd_q_bf16<F16, D, CAUSAL>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    default: return launch(attn_bwd_k_bf16<F16, D, CAUSAL>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
+    case 0: return launch(attn_fwd_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    case 1: return launch(attn_bwd_q_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    default: return launch(attn_bwd_k_bf16<F16, D, MASK>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
   }
 }
 
@@ -433,12 +430,13 @@ hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
 // which: 0 forward, 1 backward Q-tiled (dQ), 2 backward K-tiled (dK, dV)
 hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
-  if (p.f16) {
-    if (p.d == 128) return p.causal ? launch_attn_d<true, 128, true>(p, which, s) : launch_attn_d<true, 128, false>(p, which, s);
-    return p.causal ? launch_attn_d<true, 64, true>(p, which, s) : launch_attn_d<true, 64, false>(p, which, s);
-  }
-  if (p.d == 128) return p.causal ? launch_attn_d<false, 128, true>(p, which, s) : launch_attn_d<false, 128, false>(p, which, s);
-  return p.causal ? launch_attn_d<false, 64, true>(p, which, s) : launch_attn_d<false, 64, false>(p, which, s);
+  const int mask = mask_mode(p);
+#define FHOG_ATTN(F, DD)                                                            \
+  (mask == MASK_NONE ? launch_attn_d<F, DD, MASK_NONE>(p, which, s)                 \
+                     : mask == MASK_CAUSAL ? launch_attn_d<F, DD, MASK_CAUSAL>(p, which, s) : launch_attn_d<F, DD, MASK_BAND>(p, which, s))
+  if (p.f16) return p.d == 128 ? FHOG_ATTN(true, 128) : FHOG_ATTN(true, 64);
+  return p.d == 128 ? FHOG_ATTN(false, 128) : FHOG_ATTN(false, 64);
+#undef FHOG_ATTN
 }
 
 }  // namespace fhog

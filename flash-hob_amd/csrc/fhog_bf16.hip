@@ -22,7 +22,7 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-template <bool F16, int D, int PASS, bool CAUSAL>
+template <bool F16, int D, int PASS, int MASK>
 __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
@@ -31,7 +31,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   constexpr int KK = D / 16;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
@@ -61,29 +61,27 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
 
-  const int k_tiles = (p.n_k + TS - 1) / TS;
-  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;  // key tiles this workgroup visits
+  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-#pragma unroll
-  for (int x = 0; x < NT; x++) dma.issue(ring_lds + x * TILE, src[x], wave, p.n_k);
+  dma.template issue_all<NT>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
-  for (int j = 0; j < n_tiles; j++) {
-    if (j + 1 < n_tiles) {
+  for (int j = j_begin; j < j_end; j++) {
+    if (j + 1 < j_end) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-#pragma unroll
-      for (int x = 0; x < NT; x++) dma.issue(dst + x * TILE, src[x] + adv, wave, p.n_k - (j + 1) * TS);
+      dma.template issue_all<NT>(dst, TILE, src, adv, wave, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
-    // wave-uniform: the block holds masked keys (it lies on the diagonal, or reaches past the last key)
-    const bool masked = (CAUSAL && k0 == qw) || k0 + TS > p.n_k;
-    // key k0 + 8g + 4h + e is visible iff 8g + e <= lim
-    const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
-    if (!CAUSAL || k0 <= qw) {  // else every key of the tile is masked for this wave
+    const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
+    int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
+    if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
+    if (!geo.dead(k0, qw)) {  // else every key of the tile is hidden from this wave
       const char* stage = smem + (j & 1) * STAGE;
       // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
       // is cut into small pieces placed right behind the MFMAs of the same wave, where it runs in the
@@ -127,8 +125,9 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
         } else {
           e = mfma<F16>(a[c], dOb[kk], e);
           if (kk == 0 && masked) {
+            keep_branch();
 #pragma unroll
-            for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+            for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
           }
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
@@ -145,8 +144,9 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
       }
       if (PASS == 1) {
         if (masked) {
+          keep_branch();
 #pragma unroll
-          for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+          for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], dds[r], red);   // scale applied once at the end
@@ -176,7 +176,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   }
 }
 
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(256);
   const dim3 grid(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch));
@@ -184,19 +184,19 @@ hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
   hipError_t e;
   if (pass == FHOG_PASS_DD) {
     const int smem = 2 * 2 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 1, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 1, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 1, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 1, MASK>), grid, block, smem, s, p);
   } else if (pass == FHOG_PASS_B) {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 2, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 2, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 2, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 2, MASK>), grid, block, smem, s, p);
   } else {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 5, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 5, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 5, CAUSAL>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_stats_bf16<F16, D, 5, MASK>), grid, block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -214,12 +214,13 @@ hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
   if (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV) return launch_bf16_pc_pass(p, pass, s);
   if (pass != FHOG_PASS_DD && pass != FHOG_PASS_B && pass != FHOG_PASS_DD_B) return hipErrorInvalidValue;
-  if (p.f16) {
-    if (p.d == 128) return p.causal ? launch_stats_d<true, 128, true>(p, pass, s) : launch_stats_d<true, 128, false>(p, pass, s);
-    return p.causal ? launch_stats_d<true, 64, true>(p, pass, s) : launch_stats_d<true, 64, false>(p, pass, s);
-  }
-  if (p.d == 128) return p.causal ? launch_stats_d<false, 128, true>(p, pass, s) : launch_stats_d<false, 128, false>(p, pass, s);
-  return p.causal ? launch_stats_d<false, 64, true>(p, pass, s) : launch_stats_d<false, 64, false>(p, pass, s);
+  const int mask = mask_mode(p);
+#define FHOG_STATS(F, DD)                                                             \
+  (mask == MASK_NONE ? launch_stats_d<F, DD, MASK_NONE>(p, pass, s)                   \
+                     : mask == MASK_CAUSAL ? launch_stats_d<F, DD, MASK_CAUSAL>(p, pass, s) : launch_stats_d<F, DD, MASK_BAND>(p, pass, s))
+  if (p.f16) return p.d == 128 ? FHOG_STATS(true, 128) : FHOG_STATS(true, 64);
+  return p.d == 128 ? FHOG_STATS(false, 128) : FHOG_STATS(false, 64);
+#undef FHOG_STATS
 }
 
 }  // namespace fhog

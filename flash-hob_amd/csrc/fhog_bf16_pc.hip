@@ -63,7 +63,7 @@ __device__ __forceinline__ void sop_write_group(char* tile, uint32_t lo, uint32_
 
 template <bool F16, int D>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
-                                          const bf16x8_t* dOb, int lane, int lim, bool mask,
+                                          const bf16x8_t* dOb, int lane, int lo, int hi, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
   constexpr int TILE = TS * 2 * D;
   constexpr int KK = D / 16, NSTEP = 4 * KK, PF = 2, NB = PF + 1;
@@ -95,9 +95,10 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
     } else if (ph == 2) {
       dds = mfma<F16>(a[c], Qb[kk], dds);
-      if (kk == 0 && mask) {  // wave-uniform: the block lies on the diagonal or reaches past the last key
+      if (kk == 0 && mask) {  // wave-uniform: the block holds hidden keys (mask edge or end of the tensor)
+        keep_branch();
 #pragma unroll
-        for (int r = 0; r < 16; r++) pv[r] = (8 * (r / 4) + (r % 4) <= lim) ? pv[r] : 0.f;
+        for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
       }
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
@@ -141,14 +142,14 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
 }
 
 
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   using SM = PCSmem<D, false>;
   constexpr int NC = D / 32;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, CAUSAL, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
@@ -156,8 +157,9 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   const int n = lane & 31, h = lane >> 5;
   const int q0 = tile * WG_ROWS, qw = q0 + 32 * wq, qi = qw + n;
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
-  const int k_tiles = (p.n_k + TS - 1) / TS;
-  const int n_tiles = CAUSAL ? min((q0 + WG_ROWS) / TS, k_tiles) : k_tiles;
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;  // key tiles this workgroup visits
+  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
@@ -172,15 +174,15 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
     const float dsum = p.ws_d[row], dd = p.ws_dd[row], b = p.ws_b[row];
     __syncthreads();
     int sp = 0;  // ring slot of tile j
-    for (int j = 0; j <= n_tiles; j++) {
+    for (int j = j_begin; j <= j_end; j++) {
       const int k0 = j * TS;
-      if (j < n_tiles && (!CAUSAL || k0 <= qw)) {
+      if (j < j_end && !geo.dead(k0, qw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        // key k0 + 8g + 4h + e is visible iff 8g + e <= lim (diagonal block, or the block that holds the last key)
-        const int lim = min(CAUSAL && k0 == qw ? qi - k0 : TS, p.n_k - 1 - k0) - 4 * h;
-        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, lim, (CAUSAL && k0 == qw) || k0 + TS > p.n_k, c_scale_log2, l_log2,
-                          p.scale, dsum, dd, b);
+        const bool masked = geo.partial(k0, qw);
+        int lo = 0, hi = 0;  // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
+        if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
+        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, lo, hi, masked, c_scale_log2, l_log2, p.scale, dsum, dd, b);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -211,22 +213,20 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
     Dma<D> dma;
     dma.init(p.stride_kn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
-#pragma unroll
-    for (int x = 0; x < 4; x++) dma.issue(ring_lds + x * SM::TILE, src[x], wq, p.n_k);
+    dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
     dma_wait();
     __syncthreads();
     int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
-    for (int j = 0; j <= n_tiles; j++) {
-      if (j + 1 < n_tiles) {
+    for (int j = j_begin; j <= j_end; j++) {
+      if (j + 1 < j_end) {
         const uint32_t dst = ring_lds + sn * SM::STAGE;
         const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-#pragma unroll
-        for (int x = 0; x < 4; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq, p.n_k - (j + 1) * TS);
+        dma.template issue_all<4>(dst, SM::TILE, src, adv, wq, p.n_k - (j + 1) * TS);
       }
-      // block j-1: query block qb of the pair took part iff its first query is not before the tile
-      const bool act0 = j >= 1 && (!CAUSAL || (j - 1) * TS <= qw0);
-      const bool act1 = j >= 1 && (!CAUSAL || (j - 1) * TS <= qw0 + 32);
-      if (act1) {  // act0 implies act1
+      // block j-1: query block qb of the pair took part iff the tile held a key visible to it
+      const bool act0 = j > j_begin && !geo.dead((j - 1) * TS, qw0);
+      const bool act1 = j > j_begin && !geo.dead((j - 1) * TS, qw0 + 32);
+      if (act0 || act1) {
         const char* stage = smem + sc * SM::STAGE;
         const char* sop = sop_pair + ((j - 1) & 1) * SM::SOP_BUF;
         const char* bp[NCL][2];
@@ -263,14 +263,19 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
               acc_dq[0][cl] = mfma<F16>(a_op[0][0], bop[c][1], acc_dq[0][cl]);
               acc_ddo[0][cl] = mfma<F16>(a_op[0][2], bop[c][2], acc_ddo[0][cl]);
             }
-            acc_dq[1][cl] = mfma<F16>(a_op[1][0], bop[c][1], acc_dq[1][cl]);
-            acc_ddo[1][cl] = mfma<F16>(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
+            // with a plain causal mask (or none) a tile that block 0 takes part in is also one for block 1
+            if (MASK != MASK_BAND || act1) {
+              acc_dq[1][cl] = mfma<F16>(a_op[1][0], bop[c][1], acc_dq[1][cl]);
+              acc_ddo[1][cl] = mfma<F16>(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
+            }
             if (act0) {
               acc_dq[0][cl] = mfma<F16>(a_op[0][1], bop[c][0], acc_dq[0][cl]);
               acc_ddo[0][cl] = mfma<F16>(a_op[0][3], bop[c][3], acc_ddo[0][cl]);
             }
-            acc_dq[1][cl] = mfma<F16>(a_op[1][1], bop[c][0], acc_dq[1][cl]);
-            acc_ddo[1][cl] = mfma<F16>(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
+            if (MASK != MASK_BAND || act1) {
+              acc_dq[1][cl] = mfma<F16>(a_op[1][1], bop[c][0], acc_dq[1][cl]);
+              acc_ddo[1][cl] = mfma<F16>(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
+            }
             __builtin_amdgcn_sched_barrier(0);
           }
         }
@@ -303,7 +308,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 template <bool F16, int D>
 __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* ddKb,
                                           const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int lo, int hi,
-                                          bool mask, float c_scale_log2, float scale) {
+                                          bool mask, float c_scale_log2, float scale) {  // lo, hi: see StreamQueries::limits
   constexpr int TILE = TS * 2 * D;
   const int n = lane & 31, h = lane >> 5;
   const char* tQ = stage;
@@ -342,12 +347,10 @@ __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf
 #pragma unroll
     for (int j = 0; j < 4; j++) pv[4 * g + j] = __builtin_amdgcn_exp2f(s[4 * g + j] * c_scale_log2 - l4[j]);
   }
-  if (mask) {  // wave-uniform: the block lies on the diagonal or reaches past the last query
+  if (mask) {  // wave-uniform: the block holds hidden (query, key) pairs (mask edge or end of the tensor)
+    keep_branch();
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int x = 8 * (r / 4) + (r % 4);  // query row 8g + 4h + j of the tile counts iff lo <= 8g + j <= hi
-      pv[r] = (x >= lo && x <= hi) ? pv[r] : 0.f;
-    }
+    for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;  // query row 8g + 4h + j counts iff lo <= 8g + j <= hi
   }
 #pragma unroll
   for (int g = 0; g < 4; g++) {
@@ -371,7 +374,7 @@ __device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf
   sop_write<F16>(sop + 2 * SOP_TILE, ddpv, lane);
 }
 
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   using SM = PCSmem<D, true>;
@@ -387,9 +390,9 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   const int k0 = tile * WG_ROWS, kw = k0 + 32 * wq, kj = kw + n;
   const int kr = min(kj, p.n_k - 1);  // keys past the end compute on a copy of the last row; nothing of them is stored
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
-  // causal: query tiles before this workgroup's first key see none of its keys
-  const int t_begin = CAUSAL ? k0 / TS : 0;
-  const int t_end = (p.n_q + TS - 1) / TS;
+  const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
+  int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
+  geo.tile_range(k0, WG_ROWS, t_begin, t_end);
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
@@ -403,13 +406,13 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     int sp = 0;  // ring slot of tile j (slot 0 holds tile t_begin)
     for (int j = t_begin; j <= t_end; j++) {
       const int qb = j * TS;
-      if (j < t_end && (!CAUSAL || qb >= kw)) {
+      if (j < t_end && !geo.dead(qb, kw)) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
-        // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it sees key kj (diagonal block) and exists
-        const int lo = (CAUSAL && qb == kw ? kj - qb : 0) - 4 * h, hi = p.n_q - 1 - qb - 4 * h;
-        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, lo, hi, (CAUSAL && qb == kw) || qb + TS > p.n_q, c_scale_log2,
-                          p.scale);
+        const bool masked = geo.partial(qb, kw);
+        int lo = 0, hi = 0;  // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it exists and sees key kj
+        if (masked) keep_branch(), geo.limits(qb, kj, h, lo, hi);
+        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, lo, hi, masked, c_scale_log2, p.scale);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -447,8 +450,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     };
     {
       const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
-#pragma unroll
-      for (int x = 0; x < 3; x++) dma.issue(ring_lds + x * SM::TILE, src[x] + adv, wq, p.n_q - t_begin * TS);
+      dma.template issue_all<3>(ring_lds, SM::TILE, src, adv, wq, p.n_q - t_begin * TS);
       load_stat(t_begin * TS);
       store_stat(smem);
     }
@@ -460,10 +462,9 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
         const uint32_t dst = ring_lds + sn * SM::STAGE;
         const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
         load_stat((j + 1) * TS);
-#pragma unroll
-        for (int x = 0; x < 3; x++) dma.issue(dst + x * SM::TILE, src[x] + adv, wq, p.n_q - (j + 1) * TS);
+        dma.template issue_all<3>(dst, SM::TILE, src, adv, wq, p.n_q - (j + 1) * TS);
       }
-      if (j > t_begin && (!CAUSAL || (j - 1) * TS >= kw)) {
+      if (j > t_begin && !geo.dead((j - 1) * TS, kw)) {
         const char* stage = smem + sc * SM::STAGE;
         const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
         const char* bp[NC][2];
@@ -519,20 +520,20 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   }
 }
 
-template <bool F16, int D, bool CAUSAL>
+template <bool F16, int D, int MASK>
 hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(PC_THREADS);
   hipError_t e;
   if (pass == FHOG_PASS_DQ_DDO) {
     const int smem = PCSmem<D, false>::TOTAL;
-    e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep3_pc<F16, D, CAUSAL>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep3_pc<F16, D, MASK>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
   } else {
     const int smem = PCSmem<D, true>::TOTAL;
-    e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_sweep_pc<F16, D, CAUSAL>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((k_sweep_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -540,12 +541,13 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
 }  // namespace
 
 hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s) {
-  if (p.f16) {
-    if (p.d == 128) return p.causal ? launch_pc_d<true, 128, true>(p, pass, s) : launch_pc_d<true, 128, false>(p, pass, s);
-    return p.causal ? launch_pc_d<true, 64, true>(p, pass, s) : launch_pc_d<true, 64, false>(p, pass, s);
-  }
-  if (p.d == 128) return p.causal ? launch_pc_d<false, 128, true>(p, pass, s) : launch_pc_d<false, 128, false>(p, pass, s);
-  return p.causal ? launch_pc_d<false, 64, true>(p, pass, s) : launch_pc_d<false, 64, false>(p, pass, s);
+  const int mask = mask_mode(p);
+#define FHOG_PC(F, DD)                                                          \
+  (mask == MASK_NONE ? launch_pc_d<F, DD, MASK_NONE>(p, pass, s)                \
+                     : mask == MASK_CAUSAL ? launch_pc_d<F, DD, MASK_CAUSAL>(p, pass, s) : launch_pc_d<F, DD, MASK_BAND>(p, pass, s))
+  if (p.f16) return p.d == 128 ? FHOG_PC(true, 128) : FHOG_PC(true, 64);
+  return p.d == 128 ? FHOG_PC(false, 128) : FHOG_PC(false, 64);
+#undef FHOG_PC
 }
 
 }  // namespace fhog

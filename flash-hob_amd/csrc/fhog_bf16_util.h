@@ -129,16 +129,34 @@ struct Dma {
 #pragma unroll
     for (int u = 0; u < PER_WAVE; u++) voff[u] = lane_offset(u, TS);
   }
-  // tile_lds: LDS byte address of the destination tile (wave-uniform); src: first row of the source tile;
+  // tile_lds: LDS byte address of the destination tile (wave-uniform); src + adv: first row of the source tile;
   // rows_valid: rows of the tensor from that row on (>= TS for a full tile). A partial tile is filled up with copies of
   // the tensor's last row, so that no load leaves the tensor; the kernels mask those rows.
-  __device__ __forceinline__ void issue(uint32_t tile_lds, const __bf16* src, int lw, int rows_valid = TS) const {
+  // N tiles of the same rows from N tensors: tensor x goes to tile_lds + x * tile_stride and starts at src[x] + adv.
+  // ONE scalar branch decides between the precomputed offsets and the clamped ones of a partial tile, so the common
+  // case costs no vector work.
+  template <int N, int NSRC>
+  __device__ __forceinline__ void issue_all(uint32_t tile_lds, int tile_stride, const __bf16* const (&src)[NSRC], int64_t adv,
+                                            int lw, int rows_valid) const {
+    static_assert(N <= NSRC, "more tiles than tensors");
+    if (__builtin_amdgcn_readfirstlane(rows_valid) >= TS) {
 #pragma unroll
-    for (int u = 0; u < PER_WAVE; u++) {
-      const uint32_t m0 = __builtin_amdgcn_readfirstlane(tile_lds + (lw + 4 * u) * 1024);
-      const uint32_t off = rows_valid >= TS ? voff[u] : lane_offset(u, rows_valid);
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
+      for (int x = 0; x < N; x++)
+#pragma unroll
+        for (int u = 0; u < PER_WAVE; u++) issue_one(tile_lds + x * tile_stride + (lw + 4 * u) * 1024, voff[u], src[x] + adv);
+    } else {
+      uint32_t off[PER_WAVE];
+#pragma unroll
+      for (int u = 0; u < PER_WAVE; u++) off[u] = lane_offset(u, rows_valid);
+#pragma unroll
+      for (int x = 0; x < N; x++)
+#pragma unroll
+        for (int u = 0; u < PER_WAVE; u++) issue_one(tile_lds + x * tile_stride + (lw + 4 * u) * 1024, off[u], src[x] + adv);
     }
+  }
+  __device__ __forceinline__ static void issue_one(uint32_t lds, uint32_t off, const __bf16* src) {
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
   }
 };
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -156,6 +174,87 @@ __device__ __forceinline__ void load_resident(bf16x8_t* dst, const __bf16* base,
   const __bf16* p = base + (int64_t)row * ld + 8 * h;
 #pragma unroll
   for (int kk = 0; kk < D / 16; kk++) dst[kk] = *reinterpret_cast<const bf16x8_t*>(p + 16 * kk);
+}
+
+// ---- mask geometry ------------------------------------------------------------------------------------------
+// Key j is visible to query i iff 0 <= i + off - j < win (off = 0: top-left causal, off = n_k - n_q: bottom-right;
+// win >= n_q + n_k: no window), and rows past the end of a tensor never count.
+// The kernels are compiled for three mask modes, so that the common cases carry no arithmetic they do not need:
+constexpr int MASK_NONE = 0;    // only the tensor ends
+constexpr int MASK_CAUSAL = 1;  // off = 0 and no window, known at compile time (the square causal mask)
+constexpr int MASK_BAND = 2;    // off and win from the arguments
+// "Streamed" rows come in 32-row tiles starting at t0; "stationary" rows are the 32 rows of a wave starting at r0
+// (or the rows [r0, r0 + nrows) of a workgroup for the tile range).
+//
+// StreamKeys: stationary rows are queries, streamed tiles are keys (statistics sweeps, pass 3, forward, dQ).
+template <int MASK>
+struct StreamKeys {
+  int off, win, n_k;
+  __device__ __forceinline__ StreamKeys(int off_, int win_, int n_k_)
+      : off(MASK == MASK_BAND ? off_ : 0), win(MASK == MASK_BAND ? win_ : (1 << 28)), n_k(n_k_) {}
+  // tiles [lo, hi) hold a visible key for some query of [r0, r0 + nrows)
+  __device__ __forceinline__ void tile_range(int r0, int nrows, int& lo, int& hi) const {
+    const int k_tiles = (n_k + TS - 1) / TS;
+    lo = MASK == MASK_BAND ? max(0, r0 + off - win + 1) / TS : 0;
+    hi = MASK != MASK_NONE ? min(k_tiles, (r0 + nrows - 1 + off) / TS + 1) : k_tiles;
+  }
+  // no key of tile t0 is visible to any query of [r0, r0 + 32)
+  __device__ __forceinline__ bool dead(int t0, int r0) const {
+    if (MASK == MASK_NONE) return false;
+    return t0 > r0 + 31 + off || (MASK == MASK_BAND && t0 + TS - 1 < r0 + off - win + 1);
+  }
+  // some key of tile t0 is hidden from some query of [r0, r0 + 32)
+  __device__ __forceinline__ bool partial(int t0, int r0) const {
+    if (t0 + TS > n_k) return true;
+    if (MASK == MASK_NONE) return false;
+    return t0 + TS - 1 > r0 + off || (MASK == MASK_BAND && t0 < r0 + 31 + off - win + 1);
+  }
+  // key t0 + 8g + 4h + e is visible to query i iff lo <= 8g + e <= hi
+  __device__ __forceinline__ void limits(int t0, int i, int h, int& lo, int& hi) const {
+    hi = min(MASK != MASK_NONE ? i + off - t0 : TS, n_k - 1 - t0) - 4 * h;
+    lo = MASK == MASK_BAND ? i + off - win + 1 - t0 - 4 * h : -TS;
+  }
+};
+// StreamQueries: stationary rows are keys, streamed tiles are queries (pass 4, dK and dV).
+template <int MASK>
+struct StreamQueries {
+  int off, win, n_q;
+  __device__ __forceinline__ StreamQueries(int off_, int win_, int n_q_)
+      : off(MASK == MASK_BAND ? off_ : 0), win(MASK == MASK_BAND ? win_ : (1 << 28)), n_q(n_q_) {}
+  __device__ __forceinline__ void tile_range(int r0, int nrows, int& lo, int& hi) const {
+    const int q_tiles = (n_q + TS - 1) / TS;
+    lo = MASK != MASK_NONE ? max(0, r0 - off) / TS : 0;
+    hi = MASK == MASK_BAND ? (int)min((int64_t)q_tiles, ((int64_t)r0 + nrows - 1 - off + win - 1) / TS + 1) : q_tiles;
+    hi = max(hi, lo);
+  }
+  __device__ __forceinline__ bool dead(int t0, int r0) const {
+    if (MASK == MASK_NONE) return false;
+    return t0 + TS - 1 < r0 - off || (MASK == MASK_BAND && t0 > r0 + 31 - off + win - 1);
+  }
+  __device__ __forceinline__ bool partial(int t0, int r0) const {
+    if (t0 + TS > n_q) return true;
+    if (MASK == MASK_NONE) return false;
+    return t0 < r0 + 31 - off || (MASK == MASK_BAND && t0 + TS - 1 > r0 - off + win - 1);
+  }
+  // query t0 + 8g + 4h + e sees key j iff lo <= 8g + e <= hi
+  __device__ __forceinline__ void limits(int t0, int j, int h, int& lo, int& hi) const {
+    lo = MASK != MASK_NONE ? j - off - t0 - 4 * h : -TS;
+    hi = min(MASK == MASK_BAND ? j - off + win - 1 - t0 : TS, n_q - 1 - t0) - 4 * h;
+  }
+};
+// mask mode of a launch (Params or AttnParams)
+template <typename P>
+inline int mask_mode(const P& p) {
+  if (!p.causal) return MASK_NONE;
+  return (p.mask_off == 0 && p.window >= p.n_q + p.n_k) ? MASK_CAUSAL : MASK_BAND;
+}
+
+// Placed at the top of a rarely taken wave-uniform branch: keeps the compiler from turning the branch into
+// unconditional selects that every step would pay for.
+__device__ __forceinline__ void keep_branch() { asm volatile("" ::: "memory"); }
+__device__ __forceinline__ bool in_limits(int r, int lo, int hi) {  // r: register index of an S-shaped tile
+  const int x = 8 * (r / 4) + (r % 4);
+  return x >= lo && x <= hi;
 }
 
 // XCD-aware 1-D grid. Workgroup ids go round-robin over the 8 XCDs (id % 8 = XCD), each with its own L2.

@@ -38,9 +38,9 @@ struct Params {
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   int32_t batch, n_q, n_k, d;
   float scale;
-  int32_t causal;    // some mask is set; the 16-bit family takes only the top-left one (mask_off 0, no window)
+  int32_t causal;    // some mask is set
   int32_t f16;       // 16-bit tensors are fp16 (else bf16); read by the 16-bit MFMA family only
-  int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window (fp32 family)
+  int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
   int32_t window;
 };
 
@@ -59,8 +59,10 @@ struct AttnParams {
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   int32_t batch, n_q, n_k, d;
   float scale;
-  int32_t causal;
-  int32_t f16;  // tensors are fp16 (else bf16)
+  int32_t causal;    // some mask is set
+  int32_t f16;       // tensors are fp16 (else bf16)
+  int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
+  int32_t window;
 };
 
 // Launchers implemented in the kernel translation units. Each returns hipGetLastError().

@@ -44,7 +44,7 @@ class AttnArgs(Structure):
         ("dO", c_void_p), ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p), ("ws", c_void_p),
         ("batch", c_int64), ("n_q", c_int64), ("n_k", c_int64), ("d", c_int64),
         ("stride_qb", c_int64), ("stride_qn", c_int64), ("stride_kb", c_int64), ("stride_kn", c_int64),
-        ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("reserved", c_int32),
+        ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("window", c_int32),
     ]
 
 

@@ -56,12 +56,8 @@ def _scores(q, k, scale, causal, r0, n_q=None, window=None):
     return s
 
 
-def _plain_mask(causal, window, n_q, n_k) -> bool:
-    """No mask or the square causal mask without an effective window: what the 16-bit HIP kernels implement."""
-    return not causal or (n_q == n_k and (window is None or window >= n_k))
 
-
-def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
+def _hip_args(q, k, v, scale, causal, window=None) -> Optional[_lib.AttnArgs]:
     """Arguments for the HIP first-order kernels, or None when they do not cover these tensors."""
     if not (q.is_cuda and q.dtype in _HIP_DTYPES and k.dtype == v.dtype == q.dtype):
         return None
@@ -71,7 +67,8 @@ def _hip_args(q, k, v, scale, causal) -> Optional[_lib.AttnArgs]:
     a.n_k = k.shape[1]
     a.stride_qb, a.stride_qn = q.stride(0), q.stride(1)
     a.stride_kb, a.stride_kn = k.stride(0), k.stride(1)
-    a.scale, a.dtype, a.causal = float(scale), _HIP_DTYPES[q.dtype], int(bool(causal))
+    a.scale, a.dtype = float(scale), _HIP_DTYPES[q.dtype]
+    a.causal, a.window = mask_code(causal, window, q.shape[1], k.shape[1])
     return a
 
 
@@ -79,12 +76,12 @@ def _same_layout(ts) -> bool:
     return all(t.stride() == ts[0].stride() and t.stride(-1) == 1 for t in ts)
 
 
-def _attention_forward_hip(q, k, v, scale, causal):
+def _attention_forward_hip(q, k, v, scale, causal, window=None):
     """O and L from ``fhog_attn_fwd``; None when the kernels do not cover the arguments."""
     q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
     if not _same_layout([k, v]):
         k, v = k.contiguous(), v.contiguous()
-    a = _hip_args(q, k, v, scale, causal)
+    a = _hip_args(q, k, v, scale, causal, window)
     if a is None:
         return None
     L_ = _lib.lib()
@@ -98,7 +95,7 @@ def _attention_forward_hip(q, k, v, scale, causal):
     return o, lse
 
 
-def _attention_backward_hip(q, k, v, o, do, L, scale, causal):
+def _attention_backward_hip(q, k, v, o, do, L, scale, causal, window=None):
     ts_q = [t if t.stride(-1) == 1 else t.contiguous() for t in (q, o, do)]
     if not _same_layout(ts_q):
         ts_q = [t.contiguous() for t in ts_q]
@@ -106,7 +103,7 @@ def _attention_backward_hip(q, k, v, o, do, L, scale, causal):
     if not _same_layout(ts_k):
         ts_k = [t.contiguous() for t in ts_k]
     (q, o, do), (k, v) = ts_q, ts_k
-    a = _hip_args(q, k, v, scale, causal)
+    a = _hip_args(q, k, v, scale, causal, window)
     if a is None or o.dtype != q.dtype or do.dtype != q.dtype:
         return None
     L_ = _lib.lib()
@@ -145,7 +142,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, w
     mask_code(causal, window, n_q, n_k)  # raises on an inapplicable mask
     scale = d ** -0.5 if scale is None else scale
     if use_hip is not False:
-        res = _attention_forward_hip(q, k, v, scale, causal) if _plain_mask(causal, window, n_q, n_k) else None
+        res = _attention_forward_hip(q, k, v, scale, causal, window)
         if res is not None:
             return res
         if use_hip:
@@ -174,7 +171,7 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal, *, window: Optio
     batch, n_q, d = q.shape
     n_k = k.shape[1]
     if use_hip is not False:
-        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal) if _plain_mask(causal, window, n_q, n_k) else None
+        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal, window)
         if res is not None:
             return res
         if use_hip:

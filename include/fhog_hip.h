@@ -65,8 +65,7 @@ extern "C" {
 
 /* masks (fhog_bwdbwd_args.causal). With a window W > 0 key j is visible to query i iff 0 <= i' - j < W, where i' = i
    (top-left) or i' = i + n_k - n_q (bottom-right: fhog/jax_refs/jax_impl.py:110-115); W = 0 means no window.
-   The 16-bit MFMA kernels take FHOG_MASK_NONE and the plain square causal mask; every other mask runs on the
-   fp32-MFMA kernels. */
+   Both kernel families implement all of them and skip the tiles outside the band. */
 #define FHOG_MASK_NONE 0
 #define FHOG_MASK_TOP_LEFT 1     /* j <= i; needs n_q == n_k (fhog/triton_flash.py:86-92) */
 #define FHOG_MASK_BOTTOM_RIGHT 2 /* j <= i + n_k - n_q; needs n_k >= n_q, so that every query sees a key */
@@ -153,8 +152,8 @@ typedef struct fhog_attn_args {
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   float scale;
   int32_t dtype;   /* FHOG_DTYPE_BF16 | FHOG_DTYPE_FP16 */
-  int32_t causal;  /* as in fhog_bwdbwd_args */
-  int32_t reserved;
+  int32_t causal;  /* FHOG_MASK_*, as in fhog_bwdbwd_args */
+  int32_t window;  /* sliding window length in keys, 0 = none; needs a causal mask */
 } fhog_attn_args;
 
 size_t fhog_attn_args_size(void);

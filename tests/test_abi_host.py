@@ -81,7 +81,10 @@ def good_attn_args():
     (lambda a: setattr(a, "dtype", 1), 0, -3, "bf16"),
     (lambda a: setattr(a, "n_q", 200), 0, 0, ""),           # ragged lengths are fine
     (lambda a: setattr(a, "d", 32), 0, -2, "d in"),
-    (lambda a: setattr(a, "causal", 1), 0, -6, "causal"),
+    (lambda a: setattr(a, "causal", 1), 0, -6, "causal"),   # top-left needs n_q == n_k
+    (lambda a: setattr(a, "causal", 2), 0, 0, ""),
+    (lambda a: (setattr(a, "causal", 2), setattr(a, "window", 17)), 1, 0, ""),
+    (lambda a: setattr(a, "window", 17), 0, -6, "window"),
     (lambda a: setattr(a, "stride_kn", 60), 0, -4, "stride"),
     (lambda a: setattr(a, "v", 0x30008), 0, -5, "aligned"),
     (lambda a: setattr(a, "scale", float("inf")), 0, -9, "scale"),
@@ -129,7 +132,6 @@ def test_validate_accepts_good(L):
     (lambda a: (setattr(a, "causal", 2), setattr(a, "n_k", 128), setattr(a, "stride_kb", 128 * 64)), -6, "bottom-right"),
     (lambda a: setattr(a, "window", 16), -6, "window needs"),
     (lambda a: (setattr(a, "causal", 2), setattr(a, "window", -1)), -6, "window"),
-    (lambda a: (setattr(a, "causal", 2), setattr(a, "impl", 2)), -6, "impl=bf16 takes"),
     (lambda a: setattr(a, "scale", float("nan")), -9, "scale"),
 ])
 def test_validate_rejects(L, mutate, code, word):
@@ -149,18 +151,16 @@ def test_probe_rejects_bad_arguments(L):
     assert L.fhog_probe_mfma_rate(0x10000, 256, 10, 2, ctypes.byref(flops), None) == -2
 
 
-def test_masks_select_the_kernel_family(L):
-    a = good_args()                       # bf16, 256 x 512, d = 64: shape fits the 16-bit kernels
-    assert L.fhog_select_impl(ctypes.byref(a)) == 2
-    a.causal = 2                          # bottom-right on a rectangular problem: fp32-MFMA kernels
-    assert L.fhog_validate(ctypes.byref(a)) == 0
-    assert L.fhog_select_impl(ctypes.byref(a)) == 1
-    a.n_k, a.stride_kb = 256, 256 * 64    # square: bottom-right == top-left, 16-bit kernels again
-    assert L.fhog_select_impl(ctypes.byref(a)) == 2
-    a.window = 64
-    assert L.fhog_select_impl(ctypes.byref(a)) == 1
-    a.window = 256                        # a window that hides nothing
-    assert L.fhog_select_impl(ctypes.byref(a)) == 2
+def test_every_mask_runs_on_both_kernel_families(L):
+    a = good_args()                       # bf16, 256 x 512, d = 64
+    for causal, window in ((0, 0), (2, 0), (2, 64), (2, 10 ** 9)):
+        a.causal, a.window = causal, window
+        assert L.fhog_validate(ctypes.byref(a)) == 0
+        a.impl = 0
+        assert L.fhog_select_impl(ctypes.byref(a)) == 2
+        for forced in (1, 2):
+            a.impl = forced
+            assert L.fhog_validate(ctypes.byref(a)) == 0 and L.fhog_select_impl(ctypes.byref(a)) == forced
 
 
 def test_null_args(L):

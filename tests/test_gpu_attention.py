@@ -81,6 +81,28 @@ def test_fp16_forward_and_backward(causal):
         assert normalised_max_error(a, b) < 5e-3, name
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mask", [("bottom_right", None, 100, 177, 64), ("bottom_right", 40, 300, 300, 128), (True, 1, 160, 160, 64),
+                                  ("bottom_right", 33, 257, 700, 128), (True, 129, 512, 512, 128)])
+def test_band_masks_forward_and_backward(mask, dtype):
+    """Bottom-right alignment and sliding windows (fhog/jax_refs/jax_impl.py:110-115) in the HIP first-order kernels:
+    rows whose window starts in a later tile, tiles skipped on both edges of the band."""
+    import fhog
+    from fhog.attention import attention_backward
+    causal, window, n_q, n_k, d = mask
+    x = make_case(2, n_q, n_k, d, dtype, seed=28)
+    scale = d ** -0.5
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, window=window, use_hip=True)
+    o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), scale, causal, window)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(L).all()
+    assert normalised_max_error(o, o_ref) < 1e-2
+    assert (L.double().cpu() - torch.from_numpy(l_ref)).abs().max() < 2e-3
+    got = attention_backward(x["Q"], x["K"], x["V"], o, x["dO"], L, scale, causal, window=window, use_hip=True)
+    ref = first_backward(_np(x["Q"]), _np(x["K"]), _np(x["V"]), _np(x["dO"]), scale, causal, window)
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        assert normalised_max_error(a, b) < 2e-2, name
+
+
 def test_strided_rows_and_4d_input():
     """Row stride larger than d (q, k, v as slices of one packed (batch, N, 3d) tensor) and (B, H, N, d) input."""
     import fhog
