@@ -63,6 +63,28 @@ def mfma_sustained(dev):
     return res
 
 
+def other_workloads(dev, skip):
+    """The remaining reference configurations (parity-test cases, not the headline): ms per call and algorithmic TFLOP/s
+    of the same entry point, default schedule, caches from the HIP forward where it applies."""
+    import torch
+    import fhog
+    from fhog.workloads import WORKLOADS, make_inputs
+    res = {}
+    for name, w in WORKLOADS.items():
+        if name == skip:
+            continue
+        x = {n: t.flatten(0, 1).to(dev) for n, t in make_inputs(w, seed=0).items()}
+        o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)
+        plan = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale, causal=w.causal)
+        plan.run()
+        ms = event_time_ms(plan.run, 5)
+        res[name] = {"ms_per_step_no_alloc": round(ms, 4), "value": round(w.flops_algorithmic / ms / 1e9, 2),
+                     "kernel_family": {1: "fp32-mfma", 2: "bf16-mfma"}[plan.impl]}
+        del x, o, L, plan
+        torch.cuda.empty_cache()
+    return res
+
+
 def cpu_baseline(w, x_cpu, heads, repeats):
     """torch autograd double-backward (fp32, materialised, one head at a time) on the host cores."""
     import torch
@@ -172,6 +194,8 @@ def main():
                      "flops_per_launch": dom_flops, "ms_per_launch": round(per_pass[dom], 4),
                      "traffic": TRAFFIC_BYTES.get((w.name, dom))},
     }
+    if not args.workload:
+        out["other_workloads"] = other_workloads(dev, skip=w.name)
     out["mfma_sustained_tflops"] = mfma_sustained(dev)
     out["roofline"]["frac_of_sustained_random"] = round(dom_tflops / out["mfma_sustained_tflops"]["random"], 4)
     if args.cpu_heads > 0:
@@ -181,7 +205,7 @@ def main():
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), keyed by (workload, pass). None until measured for that kernel.
-TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((318.1 + 64.0) * 2 ** 20)}
+TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((320.4 + 64.0) * 2 ** 20)}
 
 if __name__ == "__main__":
     main()
