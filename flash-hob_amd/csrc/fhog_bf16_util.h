@@ -156,7 +156,7 @@ struct Dma {
   }
   __device__ __forceinline__ static void issue_one(uint32_t lds, uint32_t off, const __bf16* src) {
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory");  // M0 is reserved: the compiler keeps nothing in it
   }
 };
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
