@@ -19,6 +19,9 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// the staging loads address a 32-row tile with 32-bit byte offsets per lane: 32 rows * stride * 2 bytes must fit
+constexpr int64_t kMaxRowStride = (int64_t)1 << 24;
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // FHOG_OK or the error for a mask that does not apply to the shape
@@ -62,6 +65,7 @@ int validate(const fhog_bwdbwd_args* a) {
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
   const int vec = a->dtype == FHOG_DTYPE_FP32 ? 4 : 8;  // elements per 16 bytes
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
+  if (a->stride_qn > kMaxRowStride || a->stride_kn > kMaxRowStride) return fail(FHOG_E_STRIDE, "row stride above 2^24 elements");
   if (a->stride_qn % vec || a->stride_kn % vec || a->stride_qb % vec || a->stride_kb % vec)
     return fail(FHOG_E_STRIDE, "strides must be multiples of %d elements (16 bytes)", vec);
   if (a->batch > 1 && (a->stride_qb < a->n_q * a->stride_qn || a->stride_kb < a->n_k * a->stride_kn))
@@ -151,6 +155,7 @@ int validate_attn(const fhog_attn_args* a, int backward) {
     return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128}");
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
+  if (a->stride_qn > kMaxRowStride || a->stride_kn > kMaxRowStride) return fail(FHOG_E_STRIDE, "row stride above 2^24 elements");
   if (a->stride_qn % 8 || a->stride_kn % 8 || a->stride_qb % 8 || a->stride_kb % 8)
     return fail(FHOG_E_STRIDE, "strides must be multiples of 8 elements (16 bytes)");
   if (a->batch > 1 && (a->stride_qb < a->n_q * a->stride_qn || a->stride_kb < a->n_k * a->stride_kn))

@@ -40,7 +40,7 @@ extern "C" {
 #define FHOG_E_NULL (-1)      /* a required pointer is NULL */
 #define FHOG_E_SHAPE (-2)     /* batch/n_q/n_k/d not supported */
 #define FHOG_E_DTYPE (-3)     /* unknown dtype */
-#define FHOG_E_STRIDE (-4)    /* stride smaller than the row / not a multiple of the vector width */
+#define FHOG_E_STRIDE (-4)    /* stride smaller than the row / not a multiple of the vector width / row stride > 2^24 */
 #define FHOG_E_ALIGN (-5)     /* pointer not 16-byte aligned */
 #define FHOG_E_CAUSAL (-6)    /* mask not applicable: top-left causal with n_q != n_k, bottom-right with n_k < n_q,
                                  a window without a causal mask, or a mask the forced kernel family does not take */

@@ -86,6 +86,7 @@ def good_attn_args():
     (lambda a: (setattr(a, "causal", 2), setattr(a, "window", 17)), 1, 0, ""),
     (lambda a: setattr(a, "window", 17), 0, -6, "window"),
     (lambda a: setattr(a, "stride_kn", 60), 0, -4, "stride"),
+    (lambda a: (setattr(a, "stride_qn", (1 << 24) + 8), setattr(a, "stride_qb", 1 << 40)), 0, -4, "2^24"),
     (lambda a: setattr(a, "v", 0x30008), 0, -5, "aligned"),
     (lambda a: setattr(a, "scale", float("inf")), 0, -9, "scale"),
 ])
@@ -125,6 +126,7 @@ def test_validate_accepts_good(L):
     (lambda a: setattr(a, "schedule", 2), -3, "schedule"),
     (lambda a: setattr(a, "stride_qn", 32), -4, "stride"),
     (lambda a: setattr(a, "stride_kn", 68), -4, "multiples"),
+    (lambda a: (setattr(a, "stride_kn", (1 << 24) + 8), setattr(a, "stride_kb", 1 << 40)), -4, "2^24"),
     (lambda a: setattr(a, "stride_qb", 64), -4, "batch stride"),
     (lambda a: setattr(a, "k", 0x20004), -5, "aligned"),
     (lambda a: setattr(a, "causal", 1), -6, "top-left"),          # n_q != n_k
