@@ -261,7 +261,8 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   const bool is_fused = args->schedule == FHOG_SCHEDULE_FUSED_STATS;
   const int* order = is_fused ? fused : four;
   const int n_pass = is_fused ? 4 : 5;
-  for (int i = 0; i < n_pass; i++) {
+  // the first statistics sweep of the 16-bit family writes d_i itself: no separate launch for it
+  for (int i = impl == FHOG_IMPL_BF16 ? 1 : 0; i < n_pass; i++) {
     const int r = run_pass(args, p, impl, order[i], (hipStream_t)hip_stream);
     if (r != FHOG_OK) return r;
   }

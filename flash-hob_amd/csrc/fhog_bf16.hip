@@ -49,7 +49,22 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   const int64_t row = (int64_t)bh * p.n_q + qr;
   const float l_log2 = p.lse[row] * kLog2e;
   const float c_scale_log2 = p.scale * kLog2e;
-  const float dsum = PASS != 1 ? p.ws_d[row] : 0.f;
+  float dsum = 0.f;
+  if (PASS == 2) {
+    dsum = p.ws_d[row];
+  } else {
+    // The first statistics sweep of a chain also produces d_i = sum_c O_ic dO_ic (fhog/triton_bwdbwd.py:580) for the
+    // sweeps behind it: each lane holds half of its query's row of O and dO, one cross-half shuffle completes the sum.
+    bf16x8_t Ob[KK];
+    load_resident<D>(Ob, (const __bf16*)p.o + qoff, p.stride_qn, qr, h);
+    if (PASS == 1) load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qr, h);
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(to_f32<F16>(Ob[kk][e]), to_f32<F16>(dOb[kk][e]), dsum);
+    dsum += __shfl_xor(dsum, 32);
+    if (h == 0 && qi < p.n_q) p.ws_d[row] = dsum;
+  }
   const float dd = PASS == 2 ? p.ws_dd[row] : 0.f;
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
   // All register loads land here. The staging loads below are issued from inline asm, which the compiler's

@@ -71,6 +71,13 @@ __device__ __forceinline__ uint16_t to_elem(float x) {
   else return __builtin_bit_cast(uint16_t, (__bf16)x);
 }
 
+// element of a 16-bit carrier vector (bf16 bits, or fp16 bits when F16) as fp32
+template <bool F16>
+__device__ __forceinline__ float to_f32(__bf16 x) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, x);
+  else return (float)x;
+}
+
 // ---- S-shaped bf16 operand tiles handed from producer to consumer waves through LDS ------------
 // 32 stationary rows x 32 streamed rows, 64 bytes per row, 16-byte chunks XOR-swizzled by (row>>2)&3.
 constexpr int SOP_TILE = 32 * 64;

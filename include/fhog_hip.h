@@ -50,7 +50,9 @@ extern "C" {
 
 /* pass ids for fhog_bwdbwd_pass */
 #define FHOG_PASS_D 0      /* d_i  = sum_c O_ic dO_ic                         (fhog/triton_bwdbwd.py:580)     */
-#define FHOG_PASS_DD 1     /* dd_i = sum_j ddS_ij P_ij                        (fhog/triton_bwdbwd.py:185-211) */
+#define FHOG_PASS_DD 1     /* dd_i = sum_j ddS_ij P_ij                        (fhog/triton_bwdbwd.py:185-211);
+                              the 16-bit kernels of passes 1 and 5 also write d_i, so fhog_bwdbwd launches pass 0
+                              only for the fp32-MFMA family */
 #define FHOG_PASS_B 2      /* b_i  = sum_j dP'_ij P_ij                        (fhog/triton_bwdbwd.py:217-251) */
 #define FHOG_PASS_DQ_DDO 3 /* dQ2 = dS ddK + dS' K ; ddO = P ddV + ddP V      (fhog/triton_bwdbwd.py:257-313) */
 #define FHOG_PASS_DK_DV 4  /* dK2 = dS^T ddQ + dS'^T Q ; dV2 = ddP^T dO       (fhog/triton_bwdbwd.py:467-535) */
