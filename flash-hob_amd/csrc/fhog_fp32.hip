@@ -1,20 +1,27 @@
 // fp32-MFMA kernels of the attention double-backward: every product and every
-// intermediate in fp32 (v_mfma_f32_32x32x2_f32). This family serves fp32 inputs (bf16
-// MFMA cannot reach 1e-4) and any shape the bf16 family does not take (ragged N, d=32).
-// One wave64 per workgroup owns a 32-row tile; the opposite side streams through LDS in
-// 32-row tiles. No atomics, nothing of shape (N_Q, N_K) leaves the chip.
+// intermediate in fp32 (v_mfma_f32_32x32x2_f32). This family serves fp32 tensors (16-bit
+// MFMA cannot reach 1e-4) and d = 32; it takes bf16 and fp16 tensors of any shape too.
+// No atomics, nothing of shape (N_Q, N_K) leaves the chip.
+//
+// One kernel template for the four sweeps. A workgroup of 1, 2 or 4 wave64 owns 32 stationary
+// rows per wave (queries in passes 1-3, keys in pass 4) and keeps their operands in registers;
+// the other side streams through LDS in 32-row tiles shared by the waves. First-level products are
+// computed with the streamed rows as M and the stationary rows as N, so a lane owns ONE stationary
+// row and its registers run over the streamed rows. Such an accumulator is, as it stands, the B
+// operand of the second-level products (contraction over the streamed rows; the A operand is read
+// from the streamed LDS tile in the same row order), so nothing S-shaped passes through LDS.
 //
 // Math per tile pair (fhog/triton_bwdbwd.py:194-202, 229-243, 266-288, 485-507):
 //   S = scale Q K^T, P = exp(S - L), dP = dO V^T, ddS = scale (ddQ K^T + Q ddK^T), E = dO ddV^T
 //   dP' = E - dP dd - ddS d + dP ddS
 //   dS = scale P (dP - d), dS' = scale P (dP' - b), ddP = P (ddS - dd)
+#include "fhog_bf16_util.h"   // XCD-aware grid decode
 #include "fhog_common.h"
 
 namespace fhog {
 namespace {
 
 constexpr int TR = 32;   // rows per tile on both sides
-constexpr int SB = 33;   // row stride (floats) of the S-shaped LDS buffers
 
 template <typename T>
 __device__ inline f32x4_t load4(const T* p);
@@ -36,296 +43,318 @@ __device__ inline f32x4_t load4<_Float16>(const _Float16* p) {
   return r;
 }
 template <typename T>
-__device__ inline void store1(T* p, float x) {
-  *p = (T)x;
+__device__ inline void store4(T* p, f32x4_t x);
+template <>
+__device__ inline void store4<float>(float* p, f32x4_t x) {
+  *reinterpret_cast<f32x4_t*>(p) = x;
+}
+template <>
+__device__ inline void store4<__bf16>(__bf16* p, f32x4_t x) {
+  bf16x4_t v = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+  *reinterpret_cast<bf16x4_t*>(p) = v;
+}
+template <>
+__device__ inline void store4<_Float16>(_Float16* p, f32x4_t x) {
+  typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4_t;
+  f16x4_t v = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+  *reinterpret_cast<f16x4_t*>(p) = v;
 }
 
-// rows row0..row0+31 of a (n, D) matrix -> LDS floats with row stride D+1; rows >= n read as 0.
+// LDS tiles: 32 rows of D floats, row stride D + 4 (rows stay 16-byte aligned; 16 consecutive rows
+// at the same column fall into 16 different 16-byte bank groups).
+template <int D>
+struct Tile {
+  static constexpr int LD = D + 4;
+  static constexpr int FLOATS = TR * LD;
+};
+
+// rows row0..row0+31 of a (n, D) matrix -> LDS tile as fp32, by all threads of the workgroup; rows >= n read as 0.
 template <typename T, int D>
-__device__ inline void load_tile(float* dst, const T* src, int64_t ld, int row0, int n, int lane) {
+__device__ inline void load_tile(float* dst, const T* src, int64_t ld, int row0, int n, int tid, int nthr) {
   constexpr int C4 = D / 4;
-  for (int v = lane; v < TR * C4; v += 64) {
+  for (int v = tid; v < TR * C4; v += nthr) {
     const int r = v / C4, c = (v % C4) * 4;
     f32x4_t x = {0.f, 0.f, 0.f, 0.f};
     if (row0 + r < n) x = load4<T>(src + (int64_t)(row0 + r) * ld + c);
-    float* d = dst + r * (D + 1) + c;
-    d[0] = x[0];
-    d[1] = x[1];
-    d[2] = x[2];
-    d[3] = x[3];
+    *reinterpret_cast<f32x4_t*>(dst + r * Tile<D>::LD + c) = x;
   }
 }
 
-// acc[m][n] += sum_c A[m][c] * B[n][c]; A, B are 32 x D LDS tiles (row stride D+1).
+// Operands of one stationary row for the first-level products. The MFMA contracts two columns per
+// instruction (k = lane / 32); the columns are dealt so that each half-wave owns whole 16-byte chunks:
+// instruction 4j + e contracts columns 8j + e (lanes 0-31) and 8j + 4 + e (lanes 32-63).
+template <typename T, int D>
+__device__ inline void load_resident(f32x4_t* dst, const T* src, int64_t ld, int row, int n, int h) {
+#pragma unroll
+  for (int j = 0; j < D / 8; j++) {
+    f32x4_t x = {0.f, 0.f, 0.f, 0.f};
+    if (row < n) x = load4<T>(src + (int64_t)row * ld + 8 * j + 4 * h);
+    dst[j] = x;
+  }
+}
+
+// acc[m][n] += sum_c A[m][c] * B[n][c]: A = streamed LDS tile (m = tile row), B = stationary row n = lane % 32.
 // Result layout: acc[r] holds (m = 8*(r/4) + 4*(lane/32) + r%4, n = lane%32).
+// The LDS operand of group j + 1 is fetched before the four MFMAs of group j and the scheduler is kept from
+// hoisting more than that: one group in flight hides the LDS latency behind 256 matrix-pipe cycles, and the
+// stationary operands need the registers.
 template <int D>
-__device__ inline f32x16_t mma_nt(f32x16_t acc, const float* A, const float* B, int lane) {
-  const float* ap = A + (lane & 31) * (D + 1) + (lane >> 5);
-  const float* bp = B + (lane & 31) * (D + 1) + (lane >> 5);
-#pragma unroll 8
-  for (int c = 0; c < D; c += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[c], bp[c], acc, 0, 0, 0);
+__device__ inline f32x16_t mma_first(f32x16_t acc, const float* A, const f32x4_t* B, int lane) {
+  const float* ap = A + (lane & 31) * Tile<D>::LD + 4 * (lane >> 5);
+  f32x4_t a = *reinterpret_cast<const f32x4_t*>(ap);
+#pragma unroll
+  for (int j = 0; j < D / 8; j++) {
+    f32x4_t nxt = a;
+    if (j + 1 < D / 8) nxt = *reinterpret_cast<const f32x4_t*>(ap + 8 * (j + 1));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], B[j][e], acc, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    a = nxt;
+  }
+  return acc;
+}
+// same with the stationary operand in an LDS tile of its own (row = lane % 32)
+template <int D>
+__device__ inline f32x16_t mma_first_lds(f32x16_t acc, const float* A, const float* B, int lane) {
+  const float* ap = A + (lane & 31) * Tile<D>::LD + 4 * (lane >> 5);
+  const float* bp = B + (lane & 31) * Tile<D>::LD + 4 * (lane >> 5);
+  f32x4_t a = *reinterpret_cast<const f32x4_t*>(ap), b = *reinterpret_cast<const f32x4_t*>(bp);
+#pragma unroll
+  for (int j = 0; j < D / 8; j++) {
+    f32x4_t na = a, nb = b;
+    if (j + 1 < D / 8) {
+      na = *reinterpret_cast<const f32x4_t*>(ap + 8 * (j + 1));
+      nb = *reinterpret_cast<const f32x4_t*>(bp + 8 * (j + 1));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    a = na;
+    b = nb;
+  }
   return acc;
 }
 
-struct TileVals {
-  f32x16_t p, ds, ds2, ddp;
-  float dd_part, b_part;
-};
-
-// Everything elementwise for one 32(query) x 32(key) tile pair. Lane owns query (lane%32);
-// register r owns key 8*(r/4) + 4*(lane/32) + r%4.  LEVEL: 1 = dd only, 2 = + b, 3 = all.
-template <int D, int LEVEL, bool CAUSAL>
-__device__ inline TileVals tile_math(const float* Qs, const float* dOs, const float* ddQs, const float* Ks,
-                                     const float* Vs, const float* ddKs, const float* ddVs, int lane, int q0,
-                                     int k0, int n_q, int n_k, float scale, float L, float dsum, float dd, float b,
-                                     int mask_off, int window) {
-  TileVals t;
-  const f32x16_t zero = {0};
-  f32x16_t s = mma_nt<D>(zero, Ks, Qs, lane);
-  f32x16_t dds = mma_nt<D>(zero, Ks, ddQs, lane);
-  dds = mma_nt<D>(dds, ddKs, Qs, lane);
-  f32x16_t dp = zero, e = zero;
-  if (LEVEL >= 2) {
-    dp = mma_nt<D>(zero, Vs, dOs, lane);
-    e = mma_nt<D>(zero, ddVs, dOs, lane);
-  }
-  const int qi = q0 + (lane & 31);
-  t.dd_part = 0.f;
-  t.b_part = 0.f;
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const int kj = k0 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-    bool valid = (qi < n_q) && (kj < n_k);
-    // band mask: key visible iff 0 <= (qi + mask_off) - kj < window (fhog/jax_refs/jax_impl.py:110-115)
-    if (CAUSAL) valid = valid && (kj <= qi + mask_off) && (qi + mask_off - kj < window);
-    const float p = valid ? expf(s[r] * scale - L) : 0.f;
-    const float ddsv = dds[r] * scale;
-    t.p[r] = p;
-    t.dd_part += p * ddsv;
-    if (LEVEL >= 2) {
-      const float dpv = dp[r];
-      const float dp2 = e[r] - dpv * dd - ddsv * dsum + dpv * ddsv;
-      t.b_part += p * dp2;
-      if (LEVEL >= 3) {
-        t.ds[r] = scale * p * (dpv - dsum);
-        t.ds2[r] = scale * p * (dp2 - b);
-        t.ddp[r] = p * (ddsv - dd);
-      }
-    }
-  }
-  return t;
-}
-
-// S-shaped register tile -> LDS buffer laid out [query][key], row stride SB.
-__device__ inline void spill_tile(float* buf, const f32x16_t& x, int lane) {
-#pragma unroll
-  for (int r = 0; r < 16; r++) buf[(lane & 31) * SB + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4)] = x[r];
-}
-
-// acc[cb][i][c] += sum_j W[i][j] * X[j][cb*32 + c]   (W: [query][key] buffer, X: 32 x D tile)
+// acc[cb][c][n] += sum_m X[m][cb*32 + c] * W[m][n], W being a first-level accumulator (m over its registers):
+// instruction 4g + e contracts the streamed rows 8g + e (lanes 0-31) and 8g + 4 + e (lanes 32-63), which is
+// where register 4g + e of W holds them.
 template <int D>
-__device__ inline void mma_wx(f32x16_t* acc, const float* W, const float* X, int lane) {
-  const float* wp = W + (lane & 31) * SB + (lane >> 5);
+__device__ inline void mma_second(f32x16_t* acc, const f32x16_t& w, const float* X, int lane) {
+  const float* xp = X + 4 * (lane >> 5) * Tile<D>::LD + (lane & 31);
+  constexpr int NG = 4 * (D / 32);   // groups of four instructions: (cb, g)
+  float a[4];
 #pragma unroll
-  for (int cb = 0; cb < D / 32; cb++) {
-    const float* xp = X + (lane >> 5) * (D + 1) + cb * 32 + (lane & 31);
-#pragma unroll 8
-    for (int j = 0; j < TR; j += 2) acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[j], xp[j * (D + 1)], acc[cb], 0, 0, 0);
+  for (int e = 0; e < 4; e++) a[e] = xp[e * Tile<D>::LD];
+#pragma unroll
+  for (int i = 0; i < NG; i++) {
+    const int cb = i / 4, g = i % 4;
+    float nxt[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      nxt[e] = (i + 1 < NG) ? xp[(8 * ((i + 1) % 4) + e) * Tile<D>::LD + ((i + 1) / 4) * 32] : 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; e++) acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], w[4 * g + e], acc[cb], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int e = 0; e < 4; e++) a[e] = nxt[e];
   }
 }
 
-// acc[cb][j][c] += sum_i W[i][j] * X[i][cb*32 + c]   (contraction over the buffer's rows)
-template <int D>
-__device__ inline void mma_wtx(f32x16_t* acc, const float* W, const float* X, int lane) {
-  const float* wp = W + (lane >> 5) * SB + (lane & 31);
-#pragma unroll
-  for (int cb = 0; cb < D / 32; cb++) {
-    const float* xp = X + (lane >> 5) * (D + 1) + cb * 32 + (lane & 31);
-#pragma unroll 8
-    for (int i = 0; i < TR; i += 2) acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(wp[i * SB], xp[i * (D + 1)], acc[cb], 0, 0, 0);
-  }
-}
-
+// acc[cb][r] holds column cb*32 + 8*(r/4) + 4*(lane/32) + r%4 of stationary row lane % 32
 template <typename T, int D>
-__device__ inline void store_acc(T* dst, int64_t ld, int row0, int n, const f32x16_t* acc, int lane) {
+__device__ inline void store_acc(T* dst, int64_t ld, int row, int n, const f32x16_t* acc, int h) {
+  if (row >= n) return;
 #pragma unroll
-  for (int cb = 0; cb < D / 32; cb++) {
+  for (int cb = 0; cb < D / 32; cb++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int row = row0 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-      if (row < n) store1<T>(dst + (int64_t)row * ld + cb * 32 + (lane & 31), acc[cb][r]);
+    for (int g = 0; g < 4; g++) {
+      const f32x4_t x = {acc[cb][4 * g], acc[cb][4 * g + 1], acc[cb][4 * g + 2], acc[cb][4 * g + 3]};
+      store4<T>(dst + (int64_t)row * ld + cb * 32 + 8 * g + 4 * h, x);
     }
-  }
 }
 
-template <int D>
-struct SmemLayout {
-  static constexpr int TILE = TR * (D + 1);
-  static constexpr int BUF = TR * SB;
-  static constexpr size_t BYTES = (size_t)(7 * TILE + 4 * BUF) * sizeof(float);
-};
-
-// Passes 1..3: one wave owns 32 query rows and sweeps all key tiles.
-template <typename T, int D, int PASS, bool CAUSAL>
-__global__ void __launch_bounds__(64) q_sweep_fp32(Params p) {
+// PASS 1: dd (Q-tiled), 2: b (Q-tiled), 3: dQ2 and ddO (Q-tiled), 4: dK2 and dV2 (K-tiled).
+template <typename T, int D, int PASS, bool MASKED>
+__global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  using SL = SmemLayout<D>;
-  float* Qs = smem;
-  float* dOs = Qs + SL::TILE;
-  float* ddQs = dOs + SL::TILE;
-  float* Ks = ddQs + SL::TILE;
-  float* Vs = Ks + SL::TILE;
-  float* ddKs = Vs + SL::TILE;
-  float* ddVs = ddKs + SL::TILE;
-  float* Wds = ddVs + SL::TILE;
-  float* Wds2 = Wds + SL::BUF;
-  float* Wddp = Wds2 + SL::BUF;
-  float* Wp = Wddp + SL::BUF;
+  constexpr bool KSIDE = PASS == 4;                          // the stationary rows are keys
+  constexpr int NT = PASS == 1 ? 2 : (KSIDE ? 3 : 4);        // streamed tensors
+  constexpr int NR = KSIDE ? 4 : (PASS == 1 ? 2 : 3);        // stationary tensors
+  constexpr bool LAST_IN_LDS = KSIDE && D == 128;            // the fourth stationary tensor does not fit the registers
+  constexpr int NREG = LAST_IN_LDS ? 3 : NR;
+  constexpr int J = D / 8, CB = D / 32, TF = Tile<D>::FLOATS;
 
-  const int lane = threadIdx.x;
-  const int q0 = blockIdx.x * TR;
-  const int bh = blockIdx.y;
+  const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nw = nthr >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int n_sta = KSIDE ? p.n_k : p.n_q, n_str = KSIDE ? p.n_q : p.n_k;
+  // All tiles of a slice on one XCD (one L2 streams the slice's other side). With a mask the work of a tile grows (or
+  // falls) with its index, so a workgroup takes tiles u and n_tiles - 1 - u in turn: every workgroup of a slice
+  // then does the same amount of work, whatever their number.
+  const int n_tiles = (n_sta + TR * nw - 1) / (TR * nw);
+  int bh, unit;
+  if (!bf16k::decode_block(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch, false, bh, unit)) return;
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
-  const T* Q = (const T*)p.q + qoff;
-  const T* dO = (const T*)p.dO + qoff;
-  const T* ddQ = (const T*)p.ddq + qoff;
-  const T* K = (const T*)p.k + koff;
-  const T* V = (const T*)p.v + koff;
-  const T* ddK = (const T*)p.ddk + koff;
-  const T* ddV = (const T*)p.ddv + koff;
+  const int64_t sta_ld = KSIDE ? p.stride_kn : p.stride_qn, str_ld = KSIDE ? p.stride_qn : p.stride_kn;
+  // stationary tensors: Q, ddQ, dO | K, ddK, V, ddV; streamed tensors: K, ddK, V, ddV | Q, ddQ, dO
+  const T* sta[4] = {(const T*)(KSIDE ? p.k : p.q) + (KSIDE ? koff : qoff), (const T*)(KSIDE ? p.ddk : p.ddq) + (KSIDE ? koff : qoff),
+                     (const T*)(KSIDE ? p.v : p.dO) + (KSIDE ? koff : qoff), (const T*)p.ddv + koff};
+  const T* str[4] = {(const T*)(KSIDE ? p.q : p.k) + (KSIDE ? qoff : koff), (const T*)(KSIDE ? p.ddq : p.ddk) + (KSIDE ? qoff : koff),
+                     (const T*)(KSIDE ? p.dO : p.v) + (KSIDE ? qoff : koff), (const T*)p.ddv + koff};
 
-  load_tile<T, D>(Qs, Q, p.stride_qn, q0, p.n_q, lane);
-  load_tile<T, D>(ddQs, ddQ, p.stride_qn, q0, p.n_q, lane);
-  if (PASS >= 2) load_tile<T, D>(dOs, dO, p.stride_qn, q0, p.n_q, lane);
+  float* tiles = smem;                           // NT streamed tiles
+  float* stat = tiles + NT * TF;                 // pass 4: L, d, dd, b of the 32 streamed queries
+  float* sta_lds = stat + (KSIDE ? 4 * TR : 0);  // pass 4, d = 128: ddV rows of each wave
+  const int64_t srow = (int64_t)bh * p.n_q;
 
-  const int qi = q0 + (lane & 31);
-  const bool qok = qi < p.n_q;
-  const int64_t row = (int64_t)bh * p.n_q + qi;
-  const float L = qok ? p.lse[row] : 0.f;
-  const float dsum = (PASS >= 2 && qok) ? p.ws_d[row] : 0.f;
-  const float dd = (PASS >= 2 && qok) ? p.ws_dd[row] : 0.f;
-  const float b = (PASS >= 3 && qok) ? p.ws_b[row] : 0.f;
+#pragma unroll 1
+  for (int half = 0; half < (MASKED ? 2 : 1); half++) {
+  const int tile = half ? n_tiles - 1 - unit : unit;
+  if (half && tile == unit) break;   // odd number of tiles: the middle one stands alone
+  const int r0 = tile * TR * nw, rw = r0 + TR * wave, ri = rw + n;
+
+  f32x4_t res[NREG][J];
+#pragma unroll
+  for (int x = 0; x < NREG; x++) load_resident<T, D>(res[x], sta[x], sta_ld, ri, n_sta, h);
+  if (LAST_IN_LDS) {
+    float* mine = sta_lds + wave * TF;
+    for (int v = lane; v < TR * (D / 4); v += 64) {
+      const int r = v / (D / 4), c = (v % (D / 4)) * 4;
+      f32x4_t x = {0.f, 0.f, 0.f, 0.f};
+      if (rw + r < n_sta) x = load4<T>(sta[3] + (int64_t)(rw + r) * sta_ld + c);
+      *reinterpret_cast<f32x4_t*>(mine + r * Tile<D>::LD + c) = x;
+    }
+  }
+
+  // row statistics of a query: per lane in passes 1-3, per register (from LDS) in pass 4
+  const bool rok = ri < n_sta;
+  float L = 0.f, dsum = 0.f, dd = 0.f, b = 0.f;
+  if (!KSIDE && rok) {
+    L = p.lse[srow + ri];
+    if (PASS >= 2) dsum = p.ws_d[srow + ri], dd = p.ws_dd[srow + ri];
+    if (PASS >= 3) b = p.ws_b[srow + ri];
+  }
 
   float red = 0.f;
-  f32x16_t acc_dq[D / 32], acc_ddo[D / 32];
+  f32x16_t acc0[CB], acc1[CB];   // dQ2, ddO | dK2, dV2
 #pragma unroll
-  for (int cb = 0; cb < D / 32; cb++) {
-    acc_dq[cb] = f32x16_t{0};
-    acc_ddo[cb] = f32x16_t{0};
+  for (int cb = 0; cb < CB; cb++) acc0[cb] = f32x16_t{0}, acc1[cb] = f32x16_t{0};
+
+  // streamed tiles that hold a visible pair for some stationary row of this workgroup; key j is visible to
+  // query i iff 0 <= i + mask_off - j < window (fhog/jax_refs/jax_impl.py:110-115)
+  const int rows = TR * nw;
+  int s_begin = 0, s_end = n_str;
+  if (MASKED) {
+    if (!KSIDE) {
+      s_end = (int)min((int64_t)n_str, (int64_t)r0 + rows + p.mask_off);
+      s_begin = (int)(max((int64_t)0, (int64_t)r0 + p.mask_off - p.window + 1) / TR * TR);
+    } else {
+      s_begin = max(0, r0 - p.mask_off) / TR * TR;
+      s_end = (int)min((int64_t)n_str, (int64_t)r0 + rows - 1 - p.mask_off + p.window);
+    }
   }
 
-  // key tiles that hold a visible key for some query of this tile
-  int k_begin = 0, k_end = p.n_k;
-  if (CAUSAL) {
-    k_end = min(p.n_k, q0 + TR + p.mask_off);
-    k_begin = max(0, q0 + p.mask_off - p.window + 1) / TR * TR;
-  }
-  for (int k0 = k_begin; k0 < k_end; k0 += TR) {
+  for (int s0 = s_begin; s0 < s_end; s0 += TR) {
     __syncthreads();
-    load_tile<T, D>(Ks, K, p.stride_kn, k0, p.n_k, lane);
-    load_tile<T, D>(ddKs, ddK, p.stride_kn, k0, p.n_k, lane);
-    if (PASS >= 2) {
-      load_tile<T, D>(Vs, V, p.stride_kn, k0, p.n_k, lane);
-      load_tile<T, D>(ddVs, ddV, p.stride_kn, k0, p.n_k, lane);
+#pragma unroll
+    for (int x = 0; x < NT; x++) load_tile<T, D>(tiles + x * TF, str[x], str_ld, s0, n_str, tid, nthr);
+    if (KSIDE) {
+      for (int t = tid; t < 4 * TR; t += nthr) {
+        const int which = t >> 5, qi = s0 + (t & 31);
+        const float* src = which == 0 ? p.lse : which == 1 ? p.ws_d : which == 2 ? p.ws_dd : p.ws_b;
+        stat[t] = qi < p.n_q ? src[srow + qi] : 0.f;
+      }
     }
     __syncthreads();
-    TileVals t = tile_math<D, PASS, CAUSAL>(Qs, dOs, ddQs, Ks, Vs, ddKs, ddVs, lane, q0, k0, p.n_q, p.n_k, p.scale, L,
-                                            dsum, dd, b, p.mask_off, p.window);
-    if (PASS == 1) red += t.dd_part;
-    if (PASS == 2) red += t.b_part;
-    if (PASS == 3) {
-      spill_tile(Wds, t.ds, lane);
-      spill_tile(Wds2, t.ds2, lane);
-      spill_tile(Wddp, t.ddp, lane);
-      spill_tile(Wp, t.p, lane);
-      __syncthreads();
-      mma_wx<D>(acc_dq, Wds, ddKs, lane);
-      mma_wx<D>(acc_dq, Wds2, Ks, lane);
-      mma_wx<D>(acc_ddo, Wddp, Vs, lane);
-      mma_wx<D>(acc_ddo, Wp, ddVs, lane);
+    // Every pair of this wave's rows with this tile hidden: nothing to add. Not at d = 128, where the extra loop
+    // edge makes the register allocator spill; there the element mask alone zeroes the block.
+    bool dead = false;
+    if (MASKED && D < 128) {
+      const int64_t q_lo = KSIDE ? s0 : rw, q_hi = (KSIDE ? s0 : rw) + TR - 1;   // queries of the block
+      const int64_t k_lo = KSIDE ? rw : s0, k_hi = (KSIDE ? rw : s0) + TR - 1;   // keys of the block
+      dead = k_lo > q_hi + p.mask_off || q_lo + p.mask_off - k_hi >= p.window;
     }
+    if (dead) continue;
+
+    const f32x16_t zero = {0};
+    const float* t0 = tiles;            // K   | Q
+    const float* t1 = tiles + TF;       // ddK | ddQ
+    const float* t2 = tiles + 2 * TF;   // V   | dO
+    const float* t3 = tiles + 3 * TF;   // ddV | -
+    f32x16_t sv, dds, pv;
+    if (!KSIDE) {
+      sv = mma_first<D>(zero, t0, res[0], lane);                 // K Q^T
+      dds = mma_first<D>(zero, t0, res[1], lane);                // K ddQ^T
+      dds = mma_first<D>(dds, t1, res[0], lane);                 // + ddK Q^T
+    } else {
+      sv = mma_first<D>(zero, t0, res[0], lane);                 // Q K^T
+      dds = mma_first<D>(zero, t1, res[0], lane);                // ddQ K^T
+      dds = mma_first<D>(dds, t0, res[1], lane);                 // + Q ddK^T
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = 8 * (r / 4) + 4 * h + (r % 4);
+      const int qi = KSIDE ? s0 + m : ri, kj = KSIDE ? ri : s0 + m;
+      bool valid = qi < p.n_q && kj < p.n_k;
+      if (MASKED) valid = valid && (kj <= qi + p.mask_off) && (qi + p.mask_off - kj < p.window);
+      const float Lr = KSIDE ? stat[m] : L;
+      pv[r] = valid ? __builtin_amdgcn_exp2f((sv[r] * p.scale - Lr) * kLog2e) : 0.f;
+      dds[r] *= p.scale;
+    }
+    if (PASS == 1) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) red += pv[r] * dds[r];
+      continue;
+    }
+    f32x16_t w;
+    if (PASS >= 3) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float ddr = KSIDE ? stat[2 * TR + 8 * (r / 4) + 4 * h + (r % 4)] : dd;
+        w[r] = pv[r] * (dds[r] - ddr);                            // ddP
+      }
+      mma_second<D>(acc1, w, t2, lane);                          // ddO += ddP V | dV2 += ddP^T dO
+      if (!KSIDE) mma_second<D>(acc1, pv, t3, lane);             // ddO += P ddV
+    }
+    f32x16_t dp = KSIDE ? mma_first<D>(zero, t2, res[2], lane)    // dO V^T
+                        : mma_first<D>(zero, t2, res[2], lane);   // V dO^T
+    if (PASS >= 3) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float dr = KSIDE ? stat[TR + 8 * (r / 4) + 4 * h + (r % 4)] : dsum;
+        w[r] = p.scale * pv[r] * (dp[r] - dr);                    // dS
+      }
+      mma_second<D>(acc0, w, t1, lane);                          // dQ2 += dS ddK | dK2 += dS^T ddQ
+    }
+    f32x16_t e;
+    if (!KSIDE) e = mma_first<D>(zero, t3, res[2], lane);         // ddV dO^T
+    else if (LAST_IN_LDS) e = mma_first_lds<D>(zero, t2, sta_lds + wave * TF, lane);
+    else e = mma_first<D>(zero, t2, res[NREG - 1], lane);         // dO ddV^T
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = 8 * (r / 4) + 4 * h + (r % 4);
+      const float dr = KSIDE ? stat[TR + m] : dsum, ddr = KSIDE ? stat[2 * TR + m] : dd, br = KSIDE ? stat[3 * TR + m] : b;
+      const float dp2 = e[r] - dp[r] * ddr - dds[r] * dr + dp[r] * dds[r];
+      if (PASS == 2) red += pv[r] * dp2;
+      else w[r] = p.scale * pv[r] * (dp2 - br);                   // dS'
+    }
+    if (PASS >= 3) mma_second<D>(acc0, w, t0, lane);             // dQ2 += dS' K | dK2 += dS'^T Q
   }
 
   if (PASS == 1 || PASS == 2) {
     red += __shfl_xor(red, 32);
-    if (lane < 32 && qok) (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
+    if (h == 0 && rok) (PASS == 1 ? p.ws_dd : p.ws_b)[srow + ri] = red;
+  } else if (PASS == 3) {
+    store_acc<T, D>((T*)p.dq2 + qoff, p.stride_qn, ri, p.n_q, acc0, h);
+    store_acc<T, D>((T*)p.ddo + qoff, p.stride_qn, ri, p.n_q, acc1, h);
   } else {
-    store_acc<T, D>((T*)p.dq2 + qoff, p.stride_qn, q0, p.n_q, acc_dq, lane);
-    store_acc<T, D>((T*)p.ddo + qoff, p.stride_qn, q0, p.n_q, acc_ddo, lane);
+    store_acc<T, D>((T*)p.dk2 + koff, p.stride_kn, ri, p.n_k, acc0, h);
+    store_acc<T, D>((T*)p.dv2 + koff, p.stride_kn, ri, p.n_k, acc1, h);
   }
-}
-
-// Pass 4: one wave owns 32 key rows and sweeps all query tiles.
-template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(64) k_sweep_fp32(Params p) {
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  using SL = SmemLayout<D>;
-  float* Qs = smem;
-  float* dOs = Qs + SL::TILE;
-  float* ddQs = dOs + SL::TILE;
-  float* Ks = ddQs + SL::TILE;
-  float* Vs = Ks + SL::TILE;
-  float* ddKs = Vs + SL::TILE;
-  float* ddVs = ddKs + SL::TILE;
-  float* Wds = ddVs + SL::TILE;
-  float* Wds2 = Wds + SL::BUF;
-  float* Wddp = Wds2 + SL::BUF;
-
-  const int lane = threadIdx.x;
-  const int k0 = blockIdx.x * TR;
-  const int bh = blockIdx.y;
-  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
-  const T* Q = (const T*)p.q + qoff;
-  const T* dO = (const T*)p.dO + qoff;
-  const T* ddQ = (const T*)p.ddq + qoff;
-  const T* K = (const T*)p.k + koff;
-  const T* V = (const T*)p.v + koff;
-  const T* ddK = (const T*)p.ddk + koff;
-  const T* ddV = (const T*)p.ddv + koff;
-
-  load_tile<T, D>(Ks, K, p.stride_kn, k0, p.n_k, lane);
-  load_tile<T, D>(Vs, V, p.stride_kn, k0, p.n_k, lane);
-  load_tile<T, D>(ddKs, ddK, p.stride_kn, k0, p.n_k, lane);
-  load_tile<T, D>(ddVs, ddV, p.stride_kn, k0, p.n_k, lane);
-
-  f32x16_t acc_dk[D / 32], acc_dv[D / 32];
-#pragma unroll
-  for (int cb = 0; cb < D / 32; cb++) {
-    acc_dk[cb] = f32x16_t{0};
-    acc_dv[cb] = f32x16_t{0};
-  }
-
-  // query tiles that hold a query seeing some key of this tile: k - mask_off <= i < k - mask_off + window
-  int q_begin = 0, q_end = p.n_q;
-  if (CAUSAL) {
-    q_begin = max(0, k0 - p.mask_off) / TR * TR;
-    q_end = (int)min((int64_t)p.n_q, (int64_t)k0 + TR - 1 - p.mask_off + p.window);
-  }
-  for (int q0 = q_begin; q0 < q_end; q0 += TR) {
-    __syncthreads();
-    load_tile<T, D>(Qs, Q, p.stride_qn, q0, p.n_q, lane);
-    load_tile<T, D>(dOs, dO, p.stride_qn, q0, p.n_q, lane);
-    load_tile<T, D>(ddQs, ddQ, p.stride_qn, q0, p.n_q, lane);
-    const int qi = q0 + (lane & 31);
-    const bool qok = qi < p.n_q;
-    const int64_t row = (int64_t)bh * p.n_q + qi;
-    const float L = qok ? p.lse[row] : 0.f;
-    const float dsum = qok ? p.ws_d[row] : 0.f;
-    const float dd = qok ? p.ws_dd[row] : 0.f;
-    const float b = qok ? p.ws_b[row] : 0.f;
-    __syncthreads();
-    TileVals t = tile_math<D, 3, CAUSAL>(Qs, dOs, ddQs, Ks, Vs, ddKs, ddVs, lane, q0, k0, p.n_q, p.n_k, p.scale, L, dsum,
-                                         dd, b, p.mask_off, p.window);
-    spill_tile(Wds, t.ds, lane);
-    spill_tile(Wds2, t.ds2, lane);
-    spill_tile(Wddp, t.ddp, lane);
-    __syncthreads();
-    mma_wtx<D>(acc_dk, Wds, ddQs, lane);
-    mma_wtx<D>(acc_dk, Wds2, Qs, lane);
-    mma_wtx<D>(acc_dv, Wddp, dOs, lane);
-  }
-  store_acc<T, D>((T*)p.dk2 + koff, p.stride_kn, k0, p.n_k, acc_dk, lane);
-  store_acc<T, D>((T*)p.dv2 + koff, p.stride_kn, k0, p.n_k, acc_dv, lane);
+  }  // half
 }
 
 // Pass 0: d_i = sum_c O_ic dO_ic  (fhog/triton_bwdbwd.py:580), fp32 result. 16 lanes per row.
@@ -352,36 +381,42 @@ __global__ void __launch_bounds__(256) rowdot_kernel(Params p) {
   if (r < rows && sub == 0) p.ws_d[r] = acc;
 }
 
+// waves per workgroup: 4 when that still gives every CU a workgroup, else fewer rows per workgroup
+// (with a mask a workgroup takes two tiles)
+inline int waves_per_group(int64_t n_rows, int64_t batch, bool masked) {
+  for (int nw = 4; nw > 1; nw >>= 1) {
+    const int64_t tiles = (n_rows + TR * nw - 1) / (TR * nw);
+    if ((masked ? (tiles + 1) / 2 : tiles) * batch >= 256) return nw;
+  }
+  return 1;
+}
+
+template <typename T, int D, int PASS, bool MASKED>
+hipError_t launch_sweep(const Params& p, hipStream_t s) {
+  constexpr bool KSIDE = PASS == 4;
+  constexpr int NT = PASS == 1 ? 2 : (KSIDE ? 3 : 4);
+  const int64_t n_rows = KSIDE ? p.n_k : p.n_q;
+  const int nw = waves_per_group(n_rows, p.batch, MASKED);
+  size_t floats = (size_t)NT * Tile<D>::FLOATS + (KSIDE ? 4 * TR : 0);
+  if (KSIDE && D == 128) floats += (size_t)nw * Tile<D>::FLOATS;
+  const int smem = (int)(floats * sizeof(float));
+  const int n_tiles = (int)((n_rows + TR * nw - 1) / (TR * nw));
+  const dim3 grid(bf16k::grid_blocks(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch)), block(64 * nw);
+  const hipError_t e = hipFuncSetAttribute((const void*)sweep_fp32<T, D, PASS, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((sweep_fp32<T, D, PASS, MASKED>), grid, block, smem, s, p);
+  return hipGetLastError();
+}
+
 template <typename T, int D>
 hipError_t launch_pass_td(const Params& p, int pass, hipStream_t s) {
-  const size_t smem = SmemLayout<D>::BYTES;
-  const dim3 block(64);
-  const dim3 gq((p.n_q + TR - 1) / TR, p.batch), gk((p.n_k + TR - 1) / TR, p.batch);
-#define FHOG_LAUNCH(kern, grid)                                                                            \
-  do {                                                                                                     \
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
-    if (e != hipSuccess) return e;                                                                         \
-    hipLaunchKernelGGL(kern, grid, block, smem, s, p);                                                     \
-  } while (0)
-  if (p.causal) {
-    switch (pass) {
-      case FHOG_PASS_DD: FHOG_LAUNCH((q_sweep_fp32<T, D, 1, true>), gq); break;
-      case FHOG_PASS_B: FHOG_LAUNCH((q_sweep_fp32<T, D, 2, true>), gq); break;
-      case FHOG_PASS_DQ_DDO: FHOG_LAUNCH((q_sweep_fp32<T, D, 3, true>), gq); break;
-      case FHOG_PASS_DK_DV: FHOG_LAUNCH((k_sweep_fp32<T, D, true>), gk); break;
-      default: return hipErrorInvalidValue;
-    }
-  } else {
-    switch (pass) {
-      case FHOG_PASS_DD: FHOG_LAUNCH((q_sweep_fp32<T, D, 1, false>), gq); break;
-      case FHOG_PASS_B: FHOG_LAUNCH((q_sweep_fp32<T, D, 2, false>), gq); break;
-      case FHOG_PASS_DQ_DDO: FHOG_LAUNCH((q_sweep_fp32<T, D, 3, false>), gq); break;
-      case FHOG_PASS_DK_DV: FHOG_LAUNCH((k_sweep_fp32<T, D, false>), gk); break;
-      default: return hipErrorInvalidValue;
-    }
+  switch (pass) {
+    case FHOG_PASS_DD: return p.causal ? launch_sweep<T, D, 1, true>(p, s) : launch_sweep<T, D, 1, false>(p, s);
+    case FHOG_PASS_B: return p.causal ? launch_sweep<T, D, 2, true>(p, s) : launch_sweep<T, D, 2, false>(p, s);
+    case FHOG_PASS_DQ_DDO: return p.causal ? launch_sweep<T, D, 3, true>(p, s) : launch_sweep<T, D, 3, false>(p, s);
+    case FHOG_PASS_DK_DV: return p.causal ? launch_sweep<T, D, 4, true>(p, s) : launch_sweep<T, D, 4, false>(p, s);
+    default: return hipErrorInvalidValue;
   }
-#undef FHOG_LAUNCH
-  return hipGetLastError();
 }
 
 template <typename T>

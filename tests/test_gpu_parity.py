@@ -223,6 +223,29 @@ def test_bf16_fused_statistics_match_separate_passes(d, causal):
     assert normalised_max_error(fused[2], separate[2]) < 1e-3      # dd_i * sum_j P dP taken out of the sum
 
 
+@pytest.mark.parametrize("fused_stats", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(3, 333, 333, 128), (2, 100, 77, 64)])
+def test_bf16_chain_writes_row_sums_d_itself(shape, dtype, fused_stats):
+    """The 16-bit chain launches no separate kernel for d = rowsum(O * dO) (fhog/triton_bwdbwd.py:580): its first
+    statistics sweep writes it. Checked on a NaN-filled workspace against fp64 and against the stand-alone pass 0."""
+    from fhog import BwdBwdPlan
+    batch, n_q, n_k, d = shape
+    x = with_caches(make_case(batch, n_q, n_k, d, dtype, seed=21, grad_std=0.1), d ** -0.5, False)
+    plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], d ** -0.5,
+                      impl="bf16", fused_stats=fused_stats)
+    plan.ws.fill_(float("nan"))
+    plan.run()
+    torch.cuda.synchronize()
+    got = plan.ws.view(3, -1)[0].clone()
+    want = (x["O"].double() * x["dO"].double()).sum(-1).flatten()
+    assert torch.isfinite(plan.ws).all()
+    assert normalised_max_error(got, want) < 1e-5
+    plan.run(only_pass=0)
+    torch.cuda.synchronize()
+    assert normalised_max_error(plan.ws.view(3, -1)[0], got) < 1e-5
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("impl", ["bf16", "fp32"])
 @pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
