@@ -187,8 +187,9 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   constexpr int NREG = LAST_IN_LDS ? 3 : NR;
   constexpr int J = D / 8, CB = D / 32, TF = Tile<D>::FLOATS;
 
-  const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nw = nthr >> 6;
+  constexpr int nw = 4, nthr = 64 * nw;   // waves per workgroup (waves without rows still help with the loads)
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int n_sta = KSIDE ? p.n_k : p.n_q, n_str = KSIDE ? p.n_q : p.n_k;
   // All tiles of a slice on one XCD (one L2 streams the slice's other side). With a mask the work of a tile grows (or
@@ -257,18 +258,64 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
     }
   }
 
+  // Streaming: up to d = 64 the next tile is fetched into registers while this one is computed on and written to
+  // LDS behind the step (PRE f32x4 per tensor and thread); at d = 128 the registers are taken and the tile is
+  // loaded between two barriers.
+  constexpr bool PREFETCH = D <= 64;
+  constexpr int C4 = D / 4, PRE = PREFETCH ? TR * C4 / nthr : 1;
+  f32x4_t pre[NT][PRE];
+  float pre_stat = 0.f;
+  // pass 4: thread t < 128 carries statistic t / 32 (L, d, dd, b) of streamed query t % 32
+  const float* stat_src = p.lse;
+  if ((tid >> 5) == 1) stat_src = p.ws_d;
+  if ((tid >> 5) == 2) stat_src = p.ws_dd;
+  if ((tid >> 5) == 3) stat_src = p.ws_b;
+  stat_src += srow;
+  auto fetch = [&](int s0) {
+#pragma unroll
+    for (int x = 0; x < NT; x++)
+#pragma unroll
+      for (int c = 0; c < PRE; c++) {
+        const int v = tid + c * nthr, r = v / C4, col = (v % C4) * 4;
+        f32x4_t val = {0.f, 0.f, 0.f, 0.f};
+        if (s0 + r < n_str) val = load4<T>(str[x] + (int64_t)(s0 + r) * str_ld + col);
+        pre[x][c] = val;
+      }
+    if (KSIDE && tid < 4 * TR) {
+      const int qi = s0 + (tid & 31);
+      pre_stat = qi < p.n_q ? stat_src[qi] : 0.f;
+    }
+  };
+  auto publish = [&]() {
+#pragma unroll
+    for (int x = 0; x < NT; x++)
+#pragma unroll
+      for (int c = 0; c < PRE; c++) {
+        const int v = tid + c * nthr, r = v / C4, col = (v % C4) * 4;
+        *reinterpret_cast<f32x4_t*>(tiles + x * TF + r * Tile<D>::LD + col) = pre[x][c];
+      }
+    if (KSIDE && tid < 4 * TR) stat[tid] = pre_stat;
+  };
+  if (PREFETCH && s_begin < s_end) {
+    __syncthreads();   // the tiles of the other half are no longer read
+    fetch(s_begin);
+    publish();
+  }
+
   for (int s0 = s_begin; s0 < s_end; s0 += TR) {
     __syncthreads();
+    if (PREFETCH) {
+      if (s0 + TR < s_end) fetch(s0 + TR);
+    } else {
 #pragma unroll
-    for (int x = 0; x < NT; x++) load_tile<T, D>(tiles + x * TF, str[x], str_ld, s0, n_str, tid, nthr);
-    if (KSIDE) {
-      for (int t = tid; t < 4 * TR; t += nthr) {
-        const int which = t >> 5, qi = s0 + (t & 31);
-        const float* src = which == 0 ? p.lse : which == 1 ? p.ws_d : which == 2 ? p.ws_dd : p.ws_b;
-        stat[t] = qi < p.n_q ? src[srow + qi] : 0.f;
+      for (int x = 0; x < NT; x++) load_tile<T, D>(tiles + x * TF, str[x], str_ld, s0, n_str, tid, nthr);
+      if (KSIDE && tid < 4 * TR) {
+        const int qi = s0 + (tid & 31);
+        stat[tid] = qi < p.n_q ? stat_src[qi] : 0.f;
       }
+      __syncthreads();
     }
-    __syncthreads();
+    [&]() {
     // Every pair of this wave's rows with this tile hidden: nothing to add. Not at d = 128, where the extra loop
     // edge makes the register allocator spill; there the element mask alone zeroes the block.
     bool dead = false;
@@ -277,7 +324,8 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
       const int64_t k_lo = KSIDE ? rw : s0, k_hi = (KSIDE ? rw : s0) + TR - 1;   // keys of the block
       dead = k_lo > q_hi + p.mask_off || q_lo + p.mask_off - k_hi >= p.window;
     }
-    if (dead) continue;
+    if (D < 128 && rw >= n_sta) dead = true;   // a wave without rows
+    if (dead) return;
 
     const f32x16_t zero = {0};
     const float* t0 = tiles;            // K   | Q
@@ -307,7 +355,7 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
     if (PASS == 1) {
 #pragma unroll
       for (int r = 0; r < 16; r++) red += pv[r] * dds[r];
-      continue;
+      return;
     }
     f32x16_t w;
     if (PASS >= 3) {
@@ -342,6 +390,11 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
       else w[r] = p.scale * pv[r] * (dp2 - br);                   // dS'
     }
     if (PASS >= 3) mma_second<D>(acc0, w, t0, lane);             // dQ2 += dS' K | dK2 += dS'^T Q
+    }();
+    if (PREFETCH && s0 + TR < s_end) {
+      __syncthreads();   // every wave is done reading the tile
+      publish();
+    }
   }
 
   if (PASS == 1 || PASS == 2) {
@@ -381,22 +434,12 @@ __global__ void __launch_bounds__(256) rowdot_kernel(Params p) {
   if (r < rows && sub == 0) p.ws_d[r] = acc;
 }
 
-// waves per workgroup: 4 when that still gives every CU a workgroup, else fewer rows per workgroup
-// (with a mask a workgroup takes two tiles)
-inline int waves_per_group(int64_t n_rows, int64_t batch, bool masked) {
-  for (int nw = 4; nw > 1; nw >>= 1) {
-    const int64_t tiles = (n_rows + TR * nw - 1) / (TR * nw);
-    if ((masked ? (tiles + 1) / 2 : tiles) * batch >= 256) return nw;
-  }
-  return 1;
-}
-
 template <typename T, int D, int PASS, bool MASKED>
 hipError_t launch_sweep(const Params& p, hipStream_t s) {
   constexpr bool KSIDE = PASS == 4;
   constexpr int NT = PASS == 1 ? 2 : (KSIDE ? 3 : 4);
   const int64_t n_rows = KSIDE ? p.n_k : p.n_q;
-  const int nw = waves_per_group(n_rows, p.batch, MASKED);
+  constexpr int nw = 4;   // waves per workgroup: measured best at every size (the waves share the streamed tiles and their loads)
   size_t floats = (size_t)NT * Tile<D>::FLOATS + (KSIDE ? 4 * TR : 0);
   if (KSIDE && D == 128) floats += (size_t)nw * Tile<D>::FLOATS;
   const int smem = (int)(floats * sizeof(float));
