@@ -68,15 +68,26 @@ struct Tile {
   static constexpr int FLOATS = TR * LD;
 };
 
-// rows row0..row0+31 of a (n, D) matrix -> LDS tile as fp32, by all threads of the workgroup; rows >= n read as 0.
+// rows row0..row0+31 of two (n, D) matrices -> two LDS tiles as fp32, by the 256 threads of the workgroup; rows >= n
+// read as 0. All loads are issued before the first LDS write, so the step pays one memory latency, not one per chunk.
 template <typename T, int D>
-__device__ inline void load_tile(float* dst, const T* src, int64_t ld, int row0, int n, int tid, int nthr) {
-  constexpr int C4 = D / 4;
-  for (int v = tid; v < TR * C4; v += nthr) {
-    const int r = v / C4, c = (v % C4) * 4;
-    f32x4_t x = {0.f, 0.f, 0.f, 0.f};
-    if (row0 + r < n) x = load4<T>(src + (int64_t)(row0 + r) * ld + c);
-    *reinterpret_cast<f32x4_t*>(dst + r * Tile<D>::LD + c) = x;
+__device__ inline void load_tile_pair(float* dst0, float* dst1, const T* src0, const T* src1, int64_t ld, int row0, int n, int tid) {
+  constexpr int C4 = D / 4, PER = TR * C4 / 256;
+  f32x4_t x[2][PER];
+#pragma unroll
+  for (int c = 0; c < PER; c++) {
+    const int v = tid + c * 256, r = v / C4, col = (v % C4) * 4;
+    x[0][c] = x[1][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (row0 + r < n) {
+      x[0][c] = load4<T>(src0 + (int64_t)(row0 + r) * ld + col);
+      x[1][c] = load4<T>(src1 + (int64_t)(row0 + r) * ld + col);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < PER; c++) {
+    const int v = tid + c * 256, r = v / C4, col = (v % C4) * 4;
+    *reinterpret_cast<f32x4_t*>(dst0 + r * Tile<D>::LD + col) = x[0][c];
+    *reinterpret_cast<f32x4_t*>(dst1 + r * Tile<D>::LD + col) = x[1][c];
   }
 }
 
@@ -307,8 +318,8 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
     if (PREFETCH) {
       if (s0 + TR < s_end) fetch(s0 + TR);
     } else {
-#pragma unroll
-      for (int x = 0; x < NT; x++) load_tile<T, D>(tiles + x * TF, str[x], str_ld, s0, n_str, tid, nthr);
+      load_tile_pair<T, D>(tiles, tiles + TF, str[0], str[1], str_ld, s0, n_str, tid);
+      if (NT > 2) load_tile_pair<T, D>(tiles + 2 * TF, tiles + (NT - 1) * TF, str[2], str[NT - 1], str_ld, s0, n_str, tid);
       if (KSIDE && tid < 4 * TR) {
         const int qi = s0 + (tid & 31);
         stat[tid] = qi < p.n_q ? stat_src[qi] : 0.f;
