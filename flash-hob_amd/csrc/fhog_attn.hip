@@ -19,17 +19,6 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-// Transposed A operand for a B operand that is an S-shaped accumulator kept in registers: lane
-// (col = lane%32, h = lane/32) of 32-column block cb receives, for k-step t, tile rows 16t + 4h + 0..3 (first
-// read) and 16t + 8 + 4h + 0..3 (second read) at column cb*32 + col. Per-lane part of the address, s = 0 | 1.
-template <int D>
-__device__ __forceinline__ int tr_lane_off_acc(int cb, int s, int lane) {
-  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
-  const int col = cb * 32 + 16 * b + 4 * (i & 3);
-  const int r = 8 * s + 4 * h + (i >> 2);
-  return tile_off<D>(r, col >> 3) + ((col >> 2) & 1) * 8;
-}
-
 // registers 8t .. 8t+7 of an S-shaped fp32 tile as the bf16 B operand of second-level k-step t
 template <bool F16>
 __device__ __forceinline__ bf16x8_t pack_operand(const f32x16_t& x, int t) {

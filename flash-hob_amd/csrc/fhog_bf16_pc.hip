@@ -45,20 +45,10 @@ struct PCSmem {
 //   tail                                          dS' = P E + z     [= P (E + dP (ddS - dd) - ddS d - b)]
 // LDS operands are fetched PF steps ahead. Results go to the operand tiles dS, dS', ddP, P.
 
-// registers 4g..4g+3 of one S-shaped tile, given as packed pairs pk[2g], pk[2g+1]
-__device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int lane) {
-  const int n = lane & 31, h = lane >> 5;
-#pragma unroll
-  for (int g = 0; g < 4; g++) {
-    u32x2_t v = {pk[2 * g], pk[2 * g + 1]};
-    *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = v;
-  }
-}
-
-// registers 4g..4g+3 only (one ds_write_b64), so that the hand-off writes can be spread over the stream
-__device__ __forceinline__ void sop_write_group(char* tile, uint32_t lo, uint32_t hi, int g, int lane) {
-  const int n = lane & 31, h = lane >> 5;
-  *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) = u32x2_t{lo, hi};
+// registers 8t .. 8t+7 of one S-shaped tile, given as packed pairs pk[4t] .. pk[4t+3]: one ds_write_b128, so that the
+// hand-off writes can be spread over the stream
+__device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int t, int lane) {
+  sop_write_step(tile, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]}, t, lane);
 }
 
 template <bool F16, int D>
@@ -109,13 +99,9 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
         us[r] = u0 * scale;
         us[r + 1] = u1 * scale;
       }
-      // a group of four registers is complete every 4 / EPK steps: hand it off right away, so that the writes
-      // travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
-      if ((EPK * (kk + 1)) % 4 == 0) {
-#pragma unroll
-        for (int g = (EPK * kk) / 4; g < (EPK * (kk + 1)) / 4; g++)
-          sop_write_group(sop + 0 * SOP_TILE, pk_ds[2 * g], pk_ds[2 * g + 1], g, lane);
-      }
+      // the eight registers of a k-step are complete every 8 / EPK steps: hand them off right away, so that the
+      // writes travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
+      if ((EPK * (kk + 1)) % 8 == 0) sop_write_pk(sop + 0 * SOP_TILE, pk_ds, (EPK * kk) / 8, lane);
     } else {
       e = mfma<F16>(a[c], dOb[kk], e);
 #pragma unroll
@@ -125,12 +111,9 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
         vv[r] = pv[r] * __builtin_fmaf(dds[r], us[r], -vv[r]);              // z
         vv[r + 1] = pv[r + 1] * __builtin_fmaf(dds[r + 1], us[r + 1], -vv[r + 1]);
       }
-      if ((EPK * (kk + 1)) % 4 == 0) {
-#pragma unroll
-        for (int g = (EPK * kk) / 4; g < (EPK * (kk + 1)) / 4; g++) {
-          sop_write_group(sop + 2 * SOP_TILE, pk_ddp[2 * g], pk_ddp[2 * g + 1], g, lane);
-          sop_write_group(sop + 3 * SOP_TILE, pk_p[2 * g], pk_p[2 * g + 1], g, lane);
-        }
+      if ((EPK * (kk + 1)) % 8 == 0) {
+        sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, (EPK * kk) / 8, lane);
+        sop_write_pk(sop + 3 * SOP_TILE, pk_p, (EPK * kk) / 8, lane);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -138,7 +121,8 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
 #pragma unroll
   for (int r = 0; r < 16; r += 2)
     pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
-  sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, lane);
+  sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 0, lane);
+  sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 1, lane);
 }
 
 
@@ -204,8 +188,8 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
     int troff[2][2];
 #pragma unroll
     for (int cl = 0; cl < 2; cl++) {
-      troff[cl][0] = tr_lane_off<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 0, lane);
-      troff[cl][1] = tr_lane_off<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 1, lane);
+      troff[cl][0] = tr_lane_off_acc<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 0, lane);
+      troff[cl][1] = tr_lane_off_acc<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 1, lane);
     }
     constexpr int NCL = (D == 128) ? 2 : 1;  // 32-column blocks per consumer wave
     const int qw0 = q0 + 64 * qp;            // first query of the pair
@@ -431,8 +415,8 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     int troff[NC][2];
 #pragma unroll
     for (int cb = 0; cb < NC; cb++) {
-      troff[cb][0] = tr_lane_off<D>(cb, 0, lane);
-      troff[cb][1] = tr_lane_off<D>(cb, 1, lane);
+      troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+      troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
     }
     Dma<D> dma;
     dma.init(p.stride_qn, wq, lane);

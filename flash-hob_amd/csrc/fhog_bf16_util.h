@@ -28,20 +28,22 @@ __device__ __forceinline__ bf16x8_t lds_read128(const char* smem, int off) {
   return *reinterpret_cast<const bf16x8_t*>(smem + off);
 }
 
-// Transposed (second-level) operand of the 32-column block `cb`, read with ds_read_b64_tr_b16: lane
-// (col = lane%32, h = lane/32) receives the 8 K-slots = tile rows 16t + 8h + 0..7 at column
-// cb*32 + col. Two 8-byte transposing reads, one per group of 4 rows; within a 16-lane group lane i
-// addresses row (i>>2), columns 4*(i&3)..+3, and receives column i of the 4 x 16 block.
-// The per-lane part of the address does not depend on t and is precomputed:
-//   tr_lane_off(cb, s) for s = 0 (rows 8h + 0..3) and s = 1 (rows 8h + 4..7); step t adds 16 rows.
+// Transposed (second-level) operand of the 32-column block `cb`, read with ds_read_b64_tr_b16 from a 32-row tile:
+// two 8-byte transposing reads, one per group of 4 rows; within a 16-lane group lane i addresses row (i>>2), columns
+// 4*(i&3)..+3, and receives column i of the 4 x 16 block. The other operand of such a contraction is always an
+// S-shaped accumulator (in registers, or handed over through an operand tile), whose k-step t holds, in lane half h,
+// the streamed rows 16t + 4h + 0..3 and then 16t + 8 + 4h + 0..3 (accumulator registers 8t .. 8t+7). So lane
+// (col = lane%32, h = lane/32) fetches rows 4h + 0..3 with the first read (s = 0) and rows 8 + 4h + 0..3 with the
+// second (s = 1) of the 16-row step, at column cb*32 + col. The per-lane part of the address does not depend on t and
+// is precomputed; step t adds 16 rows.
 template <int D>
-__device__ __forceinline__ int tr_lane_off(int cb, int s, int lane) {
+__device__ __forceinline__ int tr_lane_off_acc(int cb, int s, int lane) {
   const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5;
   const int col = cb * 32 + 16 * b + 4 * (i & 3);
-  const int r = 8 * h + 4 * s + (i >> 2);
+  const int r = 8 * s + 4 * h + (i >> 2);
   return tile_off<D>(r, col >> 3) + ((col >> 2) & 1) * 8;
 }
-// p0 / p1: stage base + tr_lane_off(cb, 0 / 1); `imm` = tensor offset + t * 16 rows (compile-time)
+// p0 / p1: stage base + tr_lane_off_acc(cb, 0 / 1); `imm` = tensor offset + t * 16 rows (compile-time)
 __device__ __forceinline__ bf16x8_t lds_read_tr_pre(const char* p0, const char* p1, int imm) {
   bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p0 + imm));
   bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)(p1 + imm));
@@ -80,17 +82,24 @@ __device__ __forceinline__ float to_f32(__bf16 x) {
 
 // ---- S-shaped bf16 operand tiles handed from producer to consumer waves through LDS ------------
 // 32 stationary rows x 32 streamed rows, 64 bytes per row, 16-byte chunks XOR-swizzled by (row>>2)&3.
+// Chunk 2t + h of row n holds accumulator registers 8t .. 8t+7 of lane (n, h), i.e. the streamed rows
+// 16t + 4h + 0..3 and 16t + 8 + 4h + 0..3: one 128-bit write per k-step on the producer side (conflict-free: 16
+// consecutive lanes hit 16 different chunk positions), one 128-bit read on the consumer side, whose other operand
+// enumerates the streamed rows in the same order (tr_lane_off_acc).
 constexpr int SOP_TILE = 32 * 64;
-// producer: registers 4g..4g+3 of an S-shaped fp32 tile (streamed rows 8g + 4h + 0..3) of stationary row n
+// producer: registers 8t .. 8t+7 of stationary row n as four packed pairs
+__device__ __forceinline__ void sop_write_step(char* tile, u32x4_t pk, int t, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+  *reinterpret_cast<u32x4_t*>(tile + n * 64 + (((2 * t + h) ^ ((n >> 2) & 3)) << 4)) = pk;
+}
 template <bool F16>
 __device__ __forceinline__ void sop_write(char* tile, const f32x16_t& x, int lane) {
-  const int n = lane & 31, h = lane >> 5;
 #pragma unroll
-  for (int g = 0; g < 4; g++)
-    *reinterpret_cast<u32x2_t*>(tile + n * 64 + ((g ^ ((n >> 2) & 3)) << 4) + 8 * h) =
-        pack4<F16>(x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]);
+  for (int t = 0; t < 2; t++)
+    sop_write_step(tile, u32x4_t{pack2<F16>(x[8 * t], x[8 * t + 1]), pack2<F16>(x[8 * t + 2], x[8 * t + 3]),
+                                 pack2<F16>(x[8 * t + 4], x[8 * t + 5]), pack2<F16>(x[8 * t + 6], x[8 * t + 7])}, t, lane);
 }
-// consumer: A operand of second-level step t: stationary row n, streamed rows 16t + 8h + 0..7
+// consumer: A operand of second-level step t: stationary row n, streamed rows in the order given above
 __device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) {
   const int n = lane & 31, h = lane >> 5;
   return *reinterpret_cast<const bf16x8_t*>(tile + n * 64 + (((2 * t + h) ^ ((n >> 2) & 3)) << 4));
