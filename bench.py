@@ -86,6 +86,21 @@ def other_workloads(dev, skip):
     return res
 
 
+def first_order(w, x, iters):
+    """The callers on either side of the path on the same workload: HIP forward (O, L) and HIP first backward
+    (dQ, dK, dV). FLOP counts: 2 products forward, 5 backward (the kernels recompute S and dP once per direction: 7)."""
+    import fhog
+    if w.d not in (64, 128) or w.dtype.itemsize != 2:
+        return None
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)
+    fwd = event_time_ms(lambda: fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal), iters)
+    bwd = event_time_ms(lambda: fhog.attention_backward(x["Q"], x["K"], x["V"], o, x["dO"], L, w.scale, w.causal), iters)
+    unit = 2 * w.d * w.pairs
+    return {"forward_ms": round(fwd, 4), "forward_tflops": round(2 * unit / fwd / 1e9, 1),
+            "backward_ms": round(bwd, 4), "backward_tflops": round(5 * unit / bwd / 1e9, 1),
+            "note": "fhog_attn_fwd / fhog_attn_bwd including output allocation; not part of `value`"}
+
+
 def cpu_baseline(w, x_cpu, heads, repeats):
     """torch autograd double-backward (fp32, materialised, one head at a time) on the host cores."""
     import torch
@@ -148,6 +163,9 @@ def main():
                                 causal=w.causal, fused_stats=True)
         for _ in range(3):
             fused.run()   # the opt-in fused statistics sweep, so that it shows in the same trace
+        for _ in range(3):  # the first-order kernels (HIP forward and first backward) on the same tensors
+            o16, L16 = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)
+            fhog.attention_backward(x["Q"], x["K"], x["V"], o16, x["dO"], L16, w.scale, w.causal)
         # a plain streaming kernel of known size (reads 256 MiB, writes 256 MiB) to calibrate byte counters
         src = torch.zeros(64 * 2 ** 20, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
@@ -158,7 +176,7 @@ def main():
 
     ms_plan = event_time_ms(plan.run, args.steps)
     per_pass = {i: event_time_ms(lambda i=i: plan.run(only_pass=i), args.steps) for i in PASS_NAMES}
-    dom = max((i for i in per_pass if i != 5), key=per_pass.get)
+    dom = max((i for i in per_pass if i != 5), key=PASS_CONTRACTIONS.get)   # the kernel with the largest share of the work
     plan_fused = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale,
                                  causal=w.causal, fused_stats=True)
     ms_fused = event_time_ms(plan_fused.run, args.steps)
@@ -197,6 +215,9 @@ def main():
     }
     if not args.workload:
         out["other_workloads"] = other_workloads(dev, skip=w.name)
+    fo = first_order(w, x, min(args.steps, 20))
+    if fo:
+        out["first_order"] = fo
     out["mfma_sustained_tflops"] = mfma_sustained(dev)
     out["roofline"]["frac_of_sustained_random"] = round(dom_tflops / out["mfma_sustained_tflops"]["random"], 4)
     if args.cpu_heads > 0:
@@ -206,7 +227,8 @@ def main():
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), keyed by (workload, pass). None until measured for that kernel.
-TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((320.4 + 64.0) * 2 ** 20)}
+TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((320.4 + 64.0) * 2 ** 20),
+                 ("cfg2_bf16_causal_4096_d128", 4): int((232.3 + 64.0) * 2 ** 20)}
 
 if __name__ == "__main__":
     main()
