@@ -24,10 +24,10 @@ for p in (ROOT / "flash-hob_amd", ROOT):
         sys.path.insert(0, str(p))
 
 PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA: 256 CU x 4096 FLOP/clk x 2.4 GHz
-PASS_NAMES = {0: "rowdot_kernel (not in the 16-bit chain: its pass 1 writes d too)", 1: "q_stats_bf16<pass 1: d, dd>",
-              2: "q_stats_bf16<pass 2: b>",
+PASS_NAMES = {0: "rowdot_kernel (not in the 16-bit chain: its pass 1 writes d too)", 1: "q_sweep_bf16<pass 1: d, dd>",
+              2: "q_sweep_bf16<pass 2: b>",
               3: "q_sweep3_pc<pass 3: dQ2, ddO>", 4: "k_sweep_pc<pass 4: dK2, dV2>",
-              5: "q_stats_bf16<fused passes 1+2: d, dd, b> (opt-in schedule)"}
+              5: "q_sweep_bf16<fused passes 1+2: d, dd, b> (opt-in schedule)"}
 # contractions each kernel needs to produce its outputs from its inputs (2*d*pairs FLOP each)
 PASS_CONTRACTIONS = {0: 0, 1: 3, 2: 5, 3: 9, 4: 8, 5: 5}
 

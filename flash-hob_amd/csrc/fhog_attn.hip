@@ -19,14 +19,6 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-// registers 8t .. 8t+7 of an S-shaped fp32 tile as the bf16 B operand of second-level k-step t
-template <bool F16>
-__device__ __forceinline__ bf16x8_t pack_operand(const f32x16_t& x, int t) {
-  u32x4_t u = {pack2<F16>(x[8 * t + 0], x[8 * t + 1]), pack2<F16>(x[8 * t + 2], x[8 * t + 3]),
-               pack2<F16>(x[8 * t + 4], x[8 * t + 5]), pack2<F16>(x[8 * t + 6], x[8 * t + 7])};
-  return __builtin_bit_cast(bf16x8_t, u);
-}
-
 // acc[cb] += tile^T (columns 32cb..32cb+31) x operand, for both k-steps and all column blocks of the tile
 template <bool F16, int D, int NOP>
 __device__ __forceinline__ void second_level(const char* const (&tile)[NOP], const int (&troff)[D / 32][2],

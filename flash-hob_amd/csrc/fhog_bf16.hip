@@ -1,21 +1,25 @@
-// bf16 MFMA kernels of the attention double-backward for gfx950 (v_mfma_f32_32x32x16_bf16,
+// 16-bit MFMA kernels of the attention double-backward for gfx950 (v_mfma_f32_32x32x16_bf16 / _f16,
 // fp32 accumulation). Four recomputation passes, no atomics, nothing of shape (N_Q, N_K)
 // leaves the chip:
-//   pass 1  dd_i        Q-tiled   (fhog/triton_bwdbwd.py:185-211)   this file
-//   pass 2  b_i         Q-tiled   (fhog/triton_bwdbwd.py:217-251)   this file
-//   pass 3  dQ2, ddO    Q-tiled   (fhog/triton_bwdbwd.py:257-313)   fhog_bf16_pc.hip
-//   pass 4  dK2, dV2    K-tiled   (fhog/triton_bwdbwd.py:467-535)   fhog_bf16_pc.hip
+//   pass 1  d_i, dd_i   Q-tiled   (fhog/triton_bwdbwd.py:580, 185-211)   q_sweep_bf16<PASS=1>
+//   pass 2  b_i         Q-tiled   (fhog/triton_bwdbwd.py:217-251)        q_sweep_bf16<PASS=2>
+//   pass 3  dQ2, ddO    Q-tiled   (fhog/triton_bwdbwd.py:257-313)        d=64: q_sweep_bf16<PASS=3>; d=128: fhog_bf16_pc.hip
+//   pass 4  dK2, dV2    K-tiled   (fhog/triton_bwdbwd.py:467-535)        d=64: k_sweep_bf16;         d=128: fhog_bf16_pc.hip
 //
-// Fused statistics sweep (PASS = 5, what fhog_bwdbwd launches): b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
+// Fused statistics sweep (PASS = 5, opt-in): b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
 // needs dd_i only as a factor of a row sum, so dd and b come out of ONE sweep with the five products of pass 2
 // and three running sums per query; the three products of a separate pass 1 are saved.
 //
-// Passes 1, 2 and 5 (row statistics only): a workgroup is 256 threads = 4 wave64 owning 128 queries,
-// two workgroups per CU. Each wave keeps its 32 query rows in registers as MFMA B operands
-// (Q, ddQ and, in pass 2, dO); K-side tiles of 32 keys stream through a two-stage LDS ring filled by
-// direct global->LDS loads. Products are computed transposed (keys = M, queries = N), so every lane
-// owns ONE query: L, d, dd are per-lane scalars and the row sum is a per-lane partial sum, reduced
-// once at the end with a single cross-half shuffle.
+// The kernels of this file are single-role: a workgroup is 256 threads = 4 wave64 owning 128 stationary rows,
+// two workgroups per CU. Each wave keeps its 32 rows in registers as MFMA B operands (Q, ddQ and, from pass 2
+// on, dO; K, ddK, V, ddV in pass 4); the other side streams through a two-stage LDS ring of 32-row tiles filled by
+// direct global->LDS loads. First-level products are computed with the streamed rows as M and the stationary
+// rows as N, so every lane owns ONE stationary row: in the Q-tiled sweeps L, d, dd, b are per-lane scalars and a
+// row sum is a per-lane partial sum, reduced once at the end with a single cross-half shuffle.
+// Passes 3 and 4 at d = 64 fit the second-level products into the same wave (256 registers): the S-shaped
+// accumulators, rounded to 16 bits, are the B operands of those products as they stand (contraction over the
+// streamed rows), the A operands are transposing reads of the staged tiles in the same row order. At d = 128
+// the output accumulators alone take 128 registers and the work is split over producer and consumer waves.
 #include "fhog_bf16_util.h"
 
 namespace fhog {
@@ -23,7 +27,7 @@ using namespace bf16k;
 namespace {
 
 template <bool F16, int D, int PASS, int MASK>
-__global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
+__global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
   constexpr int TILE = TS * 2 * D;
@@ -50,7 +54,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   const float l_log2 = p.lse[row] * kLog2e;
   const float c_scale_log2 = p.scale * kLog2e;
   float dsum = 0.f;
-  if (PASS == 2) {
+  if (PASS == 2 || PASS == 3) {
     dsum = p.ws_d[row];
   } else {
     // The first statistics sweep of a chain also produces d_i = sum_c O_ic dO_ic (fhog/triton_bwdbwd.py:580) for the
@@ -65,8 +69,23 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
     dsum += __shfl_xor(dsum, 32);
     if (h == 0 && qi < p.n_q) p.ws_d[row] = dsum;
   }
-  const float dd = PASS == 2 ? p.ws_dd[row] : 0.f;
+  const float dd = (PASS == 2 || PASS == 3) ? p.ws_dd[row] : 0.f;
+  const float b = PASS == 3 ? p.ws_b[row] : 0.f;
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
+  // PASS 3 (d = 64): the second-level products follow in the same wave, with the S-shaped tiles as B operands
+  // straight from the registers; lane = query, registers = output columns
+  constexpr int NC = D / 32;
+  f32x16_t acc_dq[NC], acc_ddo[NC];
+  int troff[NC][2];
+  if (PASS == 3) {
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      acc_dq[cb] = f32x16_t{0};
+      acc_ddo[cb] = f32x16_t{0};
+      troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+      troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+    }
+  }
   // All register loads land here. The staging loads below are issued from inline asm, which the compiler's
   // wait-count bookkeeping does not see: without this explicit wait it would keep "vmcnt(n)" waits for the
   // resident operands inside the loop, where they would stall every iteration on the tile being staged.
@@ -110,6 +129,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
       constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
       constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
       f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
+      uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];   // PASS 3: packed dS, dS', ddP, P (registers 2i, 2i+1)
       bf16x8_t a[NB];
 #pragma unroll
       for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + kTensorOfPhase[i / KK] * TILE, aoff[i % KK]);
@@ -128,10 +148,20 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
         } else if (ph == 2) {
           dds = mfma<F16>(a[c], Qb[kk], dds);
+          if (PASS == 3 && kk == 0 && masked) {
+            keep_branch();
+#pragma unroll
+            for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+          }
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 1) {
               pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+            } else if (PASS == 3) {
+              const float u = dp[r] - dsum;
+              tt[r] = __builtin_fmaf(dp[r], dd, b);   // v = dP dd + b
+              dp[r] = u;
+              us[r] = pv[r] * u;                       // dS (scale applied to the accumulator at the end)
             } else {
               us[r] = (dp[r] - dsum) * p.scale;
               if (PASS == 2) tt[r] = dp[r] * dd;
@@ -139,7 +169,7 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
           }
         } else {
           e = mfma<F16>(a[c], dOb[kk], e);
-          if (kk == 0 && masked) {
+          if (PASS != 3 && kk == 0 && masked) {
             keep_branch();
 #pragma unroll
             for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
@@ -148,6 +178,16 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 2) {
               red = __builtin_fmaf(pv[r], __builtin_fmaf(dds[r], us[r], -tt[r]), red);
+            } else if (PASS == 3) {
+              const float ddp = pv[r] * __builtin_fmaf(dds[r], p.scale, -dd);
+              tt[r] = pv[r] * __builtin_fmaf(dds[r] * dp[r], p.scale, -tt[r]);   // z = P (ddS u - v)
+              if (r & 1) {
+                pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
+                pk_ds[r / 2] = pack2<F16>(us[r - 1], us[r]);
+                pk_p[r / 2] = pack2<F16>(pv[r - 1], pv[r]);
+              } else {
+                dds[r] = ddp;
+              }
             } else {
               red_dd = __builtin_fmaf(pv[r], dds[r], red_dd);
               red_pdp = __builtin_fmaf(pv[r], dp[r], red_pdp);
@@ -168,6 +208,34 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
       } else if (PASS == 2) {
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
+      } else if (PASS == 3) {
+#pragma unroll
+        for (int r = 0; r < 16; r += 2)
+          pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], tt[r]), __builtin_fmaf(pv[r + 1], e[r + 1], tt[r + 1]));
+        // dQ2^T += ddK^T dS^T + K^T dS'^T ; ddO^T += V^T ddP^T + ddV^T P^T  (stage order K, ddK, V, ddV)
+        constexpr int NIT = 2 * NC;
+        const auto opnd = [](const uint32_t* pk, int t) {
+          return __builtin_bit_cast(bf16x8_t, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]});
+        };
+        bf16x8_t ta[2][4];
+#pragma unroll
+        for (int x = 0; x < 4; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+          const int t = it / NC, cb = it % NC, c = it & 1;
+          if (it + 1 < NIT) {
+            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+#pragma unroll
+            for (int x = 0; x < 4; x++)
+              ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          acc_dq[cb] = mfma<F16>(ta[c][1], opnd(pk_ds, t), acc_dq[cb]);
+          acc_ddo[cb] = mfma<F16>(ta[c][2], opnd(pk_ddp, t), acc_ddo[cb]);
+          acc_dq[cb] = mfma<F16>(ta[c][0], opnd(pk_ds2, t), acc_dq[cb]);
+          acc_ddo[cb] = mfma<F16>(ta[c][3], opnd(pk_p, t), acc_ddo[cb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       } else {
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], us[r] + e[r], red);
@@ -175,6 +243,22 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
     }
     dma_wait();
     __syncthreads();
+  }
+  if (PASS == 3) {
+    if (qi >= p.n_q) return;
+    uint16_t* odq = (uint16_t*)p.dq2 + qoff + (int64_t)qi * p.stride_qn;
+    uint16_t* oddo = (uint16_t*)p.ddo + qoff + (int64_t)qi * p.stride_qn;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x16_t& x = acc_dq[cb];
+        const f32x16_t& y = acc_ddo[cb];
+        *reinterpret_cast<u32x2_t*>(odq + 32 * cb + 8 * g + 4 * h) =
+            pack4<F16>(x[4 * g] * p.scale, x[4 * g + 1] * p.scale, x[4 * g + 2] * p.scale, x[4 * g + 3] * p.scale);
+        *reinterpret_cast<u32x2_t*>(oddo + 32 * cb + 8 * g + 4 * h) = pack4<F16>(y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]);
+      }
+    return;
   }
   red += __shfl_xor(red, 32);
   if (PASS == 1) red *= p.scale;
@@ -191,27 +275,231 @@ __global__ void __launch_bounds__(256, 2) q_stats_bf16(Params p) {
   }
 }
 
+// Pass 4 (dK2, dV2) at d = 64 as a single-role kernel: 256 threads = 4 waves own 128 keys (K, ddK, V, ddV rows in
+// registers), Q-side tiles of 32 queries stream through a two-stage LDS ring together with the four row statistics of
+// those queries. First-level products have the queries as M and the keys as N, so a lane owns one key and its
+// accumulator registers run over the queries; rounded to 16 bits they are the B operands of the second-level
+// products (contraction over the queries), whose A operands are transposing reads of the staged Q-side tiles.
+// At d = 64 everything fits 256 registers, so no S-shaped tile passes through LDS.
 template <bool F16, int D, int MASK>
-hipError_t launch_stats_d(const Params& p, int pass, hipStream_t s) {
+__global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
+  constexpr int STAT = 4 * TS * 4;         // L log2(e), d, dd, b of the 32 staged queries
+  constexpr int STAGE = 3 * TILE + STAT;   // Q, ddQ, dO tiles, statistics
+
+  int bh, tile;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int k0 = tile * WG_ROWS, kw = k0 + 32 * wave, kj = kw + n;
+  const int kr = min(kj, p.n_k - 1);  // keys past the end compute on a copy of the last row and store nothing
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[3] = {(const __bf16*)p.q + qoff, (const __bf16*)p.ddq + qoff, (const __bf16*)p.dO + qoff};
+  const float* stat_src = p.lse;   // thread t < 128 carries statistic t / 32 of staged query t % 32
+  if ((tid >> 5) == 1) stat_src = p.ws_d;
+  if ((tid >> 5) == 2) stat_src = p.ws_dd;
+  if ((tid >> 5) == 3) stat_src = p.ws_b;
+  stat_src += (int64_t)bh * p.n_q;
+
+  bf16x8_t Kb[KK], ddKb[KK], Vb[KK], ddVb[KK];
+  load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kr, h);
+  load_resident<D>(ddKb, (const __bf16*)p.ddk + koff, p.stride_kn, kr, h);
+  load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kr, h);
+  load_resident<D>(ddVb, (const __bf16*)p.ddv + koff, p.stride_kn, kr, h);
+  const float c_scale_log2 = p.scale * kLog2e;
+
+  int aoff[KK], troff[NC][2];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  f32x16_t acc_dk[NC], acc_dv[NC];  // dK2^T, dV2^T: lane = key, registers = columns
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    acc_dk[cb] = f32x16_t{0};
+    acc_dv[cb] = f32x16_t{0};
+  }
+  const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
+  int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
+  geo.tile_range(k0, WG_ROWS, t_begin, t_end);
+  Dma<D> dma;
+  dma.init(p.stride_qn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  float stat_reg = 0.f;
+  // The statistic is loaded (a global, not generic, load) before the staging loads of a step and first touched at
+  // the end of the step, so the wave never waits for it in between.
+  auto load_stat = [&](int q_base) {
+    if (tid < 4 * TS) stat_reg = *(global_f32_ptr)(stat_src + min(q_base + (tid & (TS - 1)), p.n_q - 1));
+  };
+  auto store_stat = [&](char* stage_base) {
+    if (tid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * TILE)[tid] = (tid < TS) ? stat_reg * kLog2e : stat_reg;
+  };
+  {
+    load_stat(t_begin * TS);
+    const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
+    dma.template issue_all<3>(ring_lds, TILE, src, adv, wave, p.n_q - t_begin * TS);
+    wait_vm0();
+    store_stat(smem);
+  }
+  __syncthreads();
+
+  for (int j = t_begin; j < t_end; j++) {
+    const int st = (j - t_begin) & 1;
+    if (j + 1 < t_end) {
+      load_stat((j + 1) * TS);
+      const uint32_t dst = ring_lds + (st ^ 1) * STAGE;
+      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
+      dma.template issue_all<3>(dst, TILE, src, adv, wave, p.n_q - (j + 1) * TS);
+    }
+    const int qb = j * TS;
+    if (!geo.dead(qb, kw)) {  // else no query of the tile sees a key of this wave
+      const char* stage = smem + st * STAGE;
+      const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
+      // five first-level products in one stream of KK k-steps; the three staged operands of step kk + 1 are
+      // fetched before the MFMAs of step kk: S = Q K^T, ddS = ddQ K^T + Q ddK^T, dP = dO V^T, E = dO ddV^T
+      f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
+      bf16x8_t a[2][3];
+#pragma unroll
+      for (int x = 0; x < 3; x++) a[0][x] = lds_read128(stage + x * TILE, aoff[0]);
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) {
+        const int c = kk & 1;
+        if (kk + 1 < KK) {
+#pragma unroll
+          for (int x = 0; x < 3; x++) a[c ^ 1][x] = lds_read128(stage + x * TILE, aoff[kk + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        s = mfma<F16>(a[c][0], Kb[kk], s);
+        dds = mfma<F16>(a[c][1], Kb[kk], dds);
+        dp = mfma<F16>(a[c][2], Vb[kk], dp);
+        dds = mfma<F16>(a[c][0], ddKb[kk], dds);
+        e = mfma<F16>(a[c][2], ddVb[kk], e);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // register 4g + i belongs to query qb + 8g + 4h + i: its statistics come from the staged arrays
+      f32x16_t pv;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 0 * TS + 8 * g + 4 * h);
+#pragma unroll
+        for (int i = 0; i < 4; i++) pv[4 * g + i] = __builtin_amdgcn_exp2f(s[4 * g + i] * c_scale_log2 - l4[i]);
+      }
+      if (geo.partial(qb, kw)) {  // wave-uniform: the block holds hidden (query, key) pairs (mask edge or tensor end)
+        int lo, hi;                // query row 8g + 4h + i of the tile counts iff lo <= 8g + i <= hi
+        geo.limits(qb, kj, h, lo, hi);
+        keep_branch();
+#pragma unroll
+        for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+      }
+      // dS -> s, dS' -> e, ddP -> dds (in place; scale on dS, dS' is applied to the accumulators at the end)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
+        const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
+        const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int r = 4 * g + i;
+          const float pr = pv[r];
+          const float ddsv = dds[r] * p.scale;
+          const float t1 = ddsv - dd4[i];
+          const float dp2 = __builtin_fmaf(-ddsv, d4[i], __builtin_fmaf(dp[r], t1, e[r]));
+          dds[r] = pr * t1;
+          s[r] = pr * (dp[r] - d4[i]);
+          e[r] = pr * (dp2 - b4[i]);
+        }
+      }
+      const bf16x8_t op_ds[2] = {pack_operand<F16>(s, 0), pack_operand<F16>(s, 1)};
+      const bf16x8_t op_ds2[2] = {pack_operand<F16>(e, 0), pack_operand<F16>(e, 1)};
+      const bf16x8_t op_ddp[2] = {pack_operand<F16>(dds, 0), pack_operand<F16>(dds, 1)};
+      // dK2^T += ddQ^T dS + Q^T dS' ; dV2^T += dO^T ddP   (stage order Q, ddQ, dO)
+      constexpr int NIT = 2 * NC;
+      bf16x8_t ta[2][3];
+#pragma unroll
+      for (int x = 0; x < 3; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+#pragma unroll
+      for (int it = 0; it < NIT; it++) {
+        const int t = it / NC, cb = it % NC, c = it & 1;
+        if (it + 1 < NIT) {
+          const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+#pragma unroll
+          for (int x = 0; x < 3; x++)
+            ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        acc_dk[cb] = mfma<F16>(ta[c][1], op_ds[t], acc_dk[cb]);
+        acc_dv[cb] = mfma<F16>(ta[c][2], op_ddp[t], acc_dv[cb]);
+        acc_dk[cb] = mfma<F16>(ta[c][0], op_ds2[t], acc_dk[cb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if (j + 1 < t_end) {
+      wait_vm0();
+      store_stat(smem + (st ^ 1) * STAGE);
+    }
+    dma_wait();
+    __syncthreads();
+  }
+  if (kj >= p.n_k) return;
+  uint16_t* odk = (uint16_t*)p.dk2 + koff + (int64_t)kj * p.stride_kn;
+  uint16_t* odv = (uint16_t*)p.dv2 + koff + (int64_t)kj * p.stride_kn;
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const f32x16_t& x = acc_dk[cb];
+      const f32x16_t& y = acc_dv[cb];
+      *reinterpret_cast<u32x2_t*>(odk + 32 * cb + 8 * g + 4 * h) =
+          pack4<F16>(x[4 * g] * p.scale, x[4 * g + 1] * p.scale, x[4 * g + 2] * p.scale, x[4 * g + 3] * p.scale);
+      *reinterpret_cast<u32x2_t*>(odv + 32 * cb + 8 * g + 4 * h) = pack4<F16>(y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]);
+    }
+}
+
+template <bool F16, int D, int MASK>
+hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(256);
   const dim3 grid(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch));
   const int tile = TS * 2 * D;
   hipError_t e;
   if (pass == FHOG_PASS_DD) {
     const int smem = 2 * 2 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 1, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 1, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 1, MASK>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 1, MASK>), grid, block, smem, s, p);
+  } else if (pass == FHOG_PASS_DK_DV) {
+    if constexpr (D == 64) {
+      const int smem = 2 * (3 * tile + 4 * TS * 4);
+      const dim3 gk(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch));
+      e = hipFuncSetAttribute((const void*)k_sweep_bf16<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e != hipSuccess) return e;
+      hipLaunchKernelGGL((k_sweep_bf16<F16, D, MASK>), gk, block, smem, s, p);
+    } else {
+      return hipErrorInvalidValue;
+    }
+  } else if (pass == FHOG_PASS_DQ_DDO) {
+    if constexpr (D == 64) {
+      const int smem = 2 * 4 * tile;
+      e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 3, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e != hipSuccess) return e;
+      hipLaunchKernelGGL((q_sweep_bf16<F16, D, 3, MASK>), grid, block, smem, s, p);
+    } else {
+      return hipErrorInvalidValue;
+    }
   } else if (pass == FHOG_PASS_B) {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 2, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 2, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 2, MASK>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 2, MASK>), grid, block, smem, s, p);
   } else {
     const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_stats_bf16<F16, D, 5, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 5, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_stats_bf16<F16, D, 5, MASK>), grid, block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 5, MASK>), grid, block, smem, s, p);
   }
   return hipGetLastError();
 }
@@ -227,15 +515,16 @@ bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
 
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
-  if (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV) return launch_bf16_pc_pass(p, pass, s);
-  if (pass != FHOG_PASS_DD && pass != FHOG_PASS_B && pass != FHOG_PASS_DD_B) return hipErrorInvalidValue;
+  // d = 128: passes 3 and 4 need the producer/consumer split to fit the registers; d = 64: single-role kernels throughout
+  if (p.d == 128 && (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV)) return launch_bf16_pc_pass(p, pass, s);
+  if (pass < FHOG_PASS_DD || pass > FHOG_PASS_DD_B) return hipErrorInvalidValue;
   const int mask = mask_mode(p);
-#define FHOG_STATS(F, DD)                                                             \
-  (mask == MASK_NONE ? launch_stats_d<F, DD, MASK_NONE>(p, pass, s)                   \
-                     : mask == MASK_CAUSAL ? launch_stats_d<F, DD, MASK_CAUSAL>(p, pass, s) : launch_stats_d<F, DD, MASK_BAND>(p, pass, s))
-  if (p.f16) return p.d == 128 ? FHOG_STATS(true, 128) : FHOG_STATS(true, 64);
-  return p.d == 128 ? FHOG_STATS(false, 128) : FHOG_STATS(false, 64);
-#undef FHOG_STATS
+#define FHOG_SINGLE(F, DD)                                                             \
+  (mask == MASK_NONE ? launch_single_d<F, DD, MASK_NONE>(p, pass, s)                   \
+                     : mask == MASK_CAUSAL ? launch_single_d<F, DD, MASK_CAUSAL>(p, pass, s) : launch_single_d<F, DD, MASK_BAND>(p, pass, s))
+  if (p.f16) return p.d == 128 ? FHOG_SINGLE(true, 128) : FHOG_SINGLE(true, 64);
+  return p.d == 128 ? FHOG_SINGLE(false, 128) : FHOG_SINGLE(false, 64);
+#undef FHOG_SINGLE
 }
 
 }  // namespace fhog

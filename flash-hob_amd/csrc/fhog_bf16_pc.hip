@@ -1,4 +1,5 @@
-// Passes 3 (dQ2, ddO) and 4 (dK2, dV2) of the bf16 MFMA family as producer/consumer kernels.
+// Passes 3 (dQ2, ddO) and 4 (dK2, dV2) of the 16-bit MFMA family at d = 128 as producer/consumer kernels (at d = 64 one
+// wave holds everything and the single-role kernels of fhog_bf16.hip are faster).
 //
 // A workgroup is 512 threads = 8 wave64, two per SIMD, owning 128 stationary rows:
 //   producers (4 waves, 32 stationary rows each): first-level products of one 32x32 block
@@ -529,8 +530,8 @@ hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s) {
 #define FHOG_PC(F, DD)                                                          \
   (mask == MASK_NONE ? launch_pc_d<F, DD, MASK_NONE>(p, pass, s)                \
                      : mask == MASK_CAUSAL ? launch_pc_d<F, DD, MASK_CAUSAL>(p, pass, s) : launch_pc_d<F, DD, MASK_BAND>(p, pass, s))
-  if (p.f16) return p.d == 128 ? FHOG_PC(true, 128) : FHOG_PC(true, 64);
-  return p.d == 128 ? FHOG_PC(false, 128) : FHOG_PC(false, 64);
+  if (p.d != 128) return hipErrorInvalidValue;   // d = 64 runs on the single-role kernels
+  return p.f16 ? FHOG_PC(true, 128) : FHOG_PC(false, 128);
 #undef FHOG_PC
 }
 

@@ -80,6 +80,14 @@ __device__ __forceinline__ float to_f32(__bf16 x) {
   else return (float)x;
 }
 
+// registers 8t .. 8t+7 of an S-shaped fp32 tile as the 16-bit B operand of second-level k-step t (in registers)
+template <bool F16>
+__device__ __forceinline__ bf16x8_t pack_operand(const f32x16_t& x, int t) {
+  u32x4_t u = {pack2<F16>(x[8 * t + 0], x[8 * t + 1]), pack2<F16>(x[8 * t + 2], x[8 * t + 3]),
+               pack2<F16>(x[8 * t + 4], x[8 * t + 5]), pack2<F16>(x[8 * t + 6], x[8 * t + 7])};
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
 // ---- S-shaped bf16 operand tiles handed from producer to consumer waves through LDS ------------
 // 32 stationary rows x 32 streamed rows, 64 bytes per row, 16-byte chunks XOR-swizzled by (row>>2)&3.
 // Chunk 2t + h of row n holds accumulator registers 8t .. 8t+7 of lane (n, h), i.e. the streamed rows
