@@ -77,8 +77,9 @@ def other_workloads(dev, skip):
         x = {n: t.flatten(0, 1).to(dev) for n, t in make_inputs(w, seed=0).items()}
         o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], w.scale, w.causal)
         plan = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale, causal=w.causal)
-        plan.run()
-        ms = event_time_ms(plan.run, 5)
+        for _ in range(10):   # the host spent seconds making the inputs: let the clocks come back up
+            plan.run()
+        ms = event_time_ms(plan.run, 20 if w.flops_algorithmic < 2e12 else 5)
         res[name] = {"ms_per_step_no_alloc": round(ms, 4), "value": round(w.flops_algorithmic / ms / 1e9, 2),
                      "kernel_family": {1: "fp32-mfma", 2: "bf16-mfma"}[plan.impl]}
         del x, o, L, plan
