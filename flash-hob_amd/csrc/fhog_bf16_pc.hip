@@ -52,9 +52,13 @@ __device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int
   sop_write_step(tile, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]}, t, lane);
 }
 
-template <bool F16, int D>
-__device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* Qb, const bf16x8_t* ddQb,
-                                          const bf16x8_t* dOb, int lane, int lo, int hi, bool mask,
+// KSIDE = false: pass 3 as described (stationary rows = queries: rs = Q, rdds = ddQ, rdp = re = dO; streamed K, V, ddK,
+// ddV). KSIDE = true: pass 4 with the same stream: stationary rows = keys (rs = K, rdds = ddK, rdp = V, re = ddV),
+// streamed Q, dO, ddQ, dO again; the resident operand goes first in the MFMA, so that a lane still owns one QUERY (a
+// streamed row) and the row statistics stay per-lane scalars, reloaded for every tile; registers run over the keys.
+template <bool F16, int D, bool KSIDE>
+__device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* rs, const bf16x8_t* rdds,
+                                          const bf16x8_t* rdp, const bf16x8_t* re, int lane, int lo, int hi, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
   constexpr int TILE = TS * 2 * D;
   constexpr int KK = D / 16, NSTEP = 4 * KK, PF = 2, NB = PF + 1;
@@ -62,8 +66,11 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
   int aoff[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
-  // stream order of the A operands: K, V, ddK, ddV (stage order is K, ddK, V, ddV)
-  constexpr int kTensorOfPhase[4] = {0, 2, 1, 3};
+  // stream order of the staged operands: K, V, ddK, ddV (stage order K, ddK, V, ddV) | Q, dO, ddQ, dO (stage order Q, ddQ, dO)
+  constexpr int kTensorOfPhase[4] = {0, 2, 1, KSIDE ? 2 : 3};
+  const auto mm = [](bf16x8_t staged, bf16x8_t resident, f32x16_t acc) {
+    return KSIDE ? mfma<F16>(resident, staged, acc) : mfma<F16>(staged, resident, acc);
+  };
   f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
   f32x16_t pv, vv, us;
   uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];
@@ -78,15 +85,15 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
     if (i + PF < NSTEP) a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
     __builtin_amdgcn_sched_barrier(0);
     if (ph == 0) {
-      s = mfma<F16>(a[c], Qb[kk], s);
-      dds = mfma<F16>(a[c], ddQb[kk], dds);
+      s = mm(a[c], rs[kk], s);
+      dds = mm(a[c], rdds[kk], dds);
     } else if (ph == 1) {
-      dp = mfma<F16>(a[c], dOb[kk], dp);
+      dp = mm(a[c], rdp[kk], dp);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
     } else if (ph == 2) {
-      dds = mfma<F16>(a[c], Qb[kk], dds);
-      if (kk == 0 && mask) {  // wave-uniform: the block holds hidden keys (mask edge or end of the tensor)
+      dds = mm(a[c], rs[kk], dds);
+      if (kk == 0 && mask) {  // wave-uniform: the block holds hidden pairs (mask edge or end of a tensor)
         keep_branch();
 #pragma unroll
         for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
@@ -104,7 +111,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       // writes travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
       if ((EPK * (kk + 1)) % 8 == 0) sop_write_pk(sop + 0 * SOP_TILE, pk_ds, (EPK * kk) / 8, lane);
     } else {
-      e = mfma<F16>(a[c], dOb[kk], e);
+      e = mm(a[c], re[kk], e);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
         pk_ddp[r / 2] = pack2<F16>(pv[r] * __builtin_fmaf(dds[r], scale, -dd), pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd));
@@ -114,7 +121,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       }
       if ((EPK * (kk + 1)) % 8 == 0) {
         sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, (EPK * kk) / 8, lane);
-        sop_write_pk(sop + 3 * SOP_TILE, pk_p, (EPK * kk) / 8, lane);
+        if (!KSIDE) sop_write_pk(sop + 3 * SOP_TILE, pk_p, (EPK * kk) / 8, lane);   // pass 4 has no use for P
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -167,7 +174,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
         const bool masked = geo.partial(k0, qw);
         int lo = 0, hi = 0;  // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
         if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
-        produce_q<F16, D>(stage, sop, Qb, ddQb, dOb, lane, lo, hi, masked, c_scale_log2, l_log2, p.scale, dsum, dd, b);
+        produce_q<F16, D, false>(stage, sop, Qb, ddQb, dOb, dOb, lane, lo, hi, masked, c_scale_log2, l_log2, p.scale, dsum, dd, b);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -290,73 +297,17 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 }
 
 // ---- pass 4 ------------------------------------------------------------------------------------------
-template <bool F16, int D>
-__device__ __forceinline__ void produce_k(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* ddKb,
-                                          const bf16x8_t* Vb, const bf16x8_t* ddVb, int lane, int lo, int hi,
-                                          bool mask, float c_scale_log2, float scale) {  // lo, hi: see StreamQueries::limits
-  constexpr int TILE = TS * 2 * D;
-  const int n = lane & 31, h = lane >> 5;
-  const char* tQ = stage;
-  const char* tddQ = stage + TILE;
-  const char* tdO = stage + 2 * TILE;
-  const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
-  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
-  bf16x8_t a[2][3];
-  {
-    const int off = tile_off<D>(n, h);
-    a[0][0] = lds_read128(tQ, off);
-    a[0][1] = lds_read128(tddQ, off);
-    a[0][2] = lds_read128(tdO, off);
-  }
-#pragma unroll
-  for (int kk = 0; kk < D / 16; kk++) {
-    const int c = kk & 1;
-    if (kk + 1 < D / 16) {
-      const int off = tile_off<D>(n, 2 * (kk + 1) + h);
-      a[c ^ 1][0] = lds_read128(tQ, off);
-      a[c ^ 1][1] = lds_read128(tddQ, off);
-      a[c ^ 1][2] = lds_read128(tdO, off);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    s = mfma<F16>(a[c][0], Kb[kk], s);
-    dds = mfma<F16>(a[c][1], Kb[kk], dds);
-    dp = mfma<F16>(a[c][2], Vb[kk], dp);
-    dds = mfma<F16>(a[c][0], ddKb[kk], dds);
-    e = mfma<F16>(a[c][2], ddVb[kk], e);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  f32x16_t pv, dsv, ds2v, ddpv;
-#pragma unroll
-  for (int g = 0; g < 4; g++) {
-    const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 0 * TS + 8 * g + 4 * h);
-#pragma unroll
-    for (int j = 0; j < 4; j++) pv[4 * g + j] = __builtin_amdgcn_exp2f(s[4 * g + j] * c_scale_log2 - l4[j]);
-  }
-  if (mask) {  // wave-uniform: the block holds hidden (query, key) pairs (mask edge or end of the tensor)
-    keep_branch();
-#pragma unroll
-    for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;  // query row 8g + 4h + j counts iff lo <= 8g + j <= hi
-  }
-#pragma unroll
-  for (int g = 0; g < 4; g++) {
-    const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
-    const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
-    const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int r = 4 * g + j;
-      const float p = pv[r];
-      const float ddsv = dds[r] * scale;
-      const float t1 = ddsv - dd4[j];
-      const float dp2 = __builtin_fmaf(-ddsv, d4[j], __builtin_fmaf(dp[r], t1, e[r]));
-      ddpv[r] = p * t1;
-      dsv[r] = p * (dp[r] - d4[j]);
-      ds2v[r] = p * (dp2 - b4[j]);
-    }
-  }
-  sop_write<F16>(sop + 0 * SOP_TILE, dsv, lane);
-  sop_write<F16>(sop + 1 * SOP_TILE, ds2v, lane);
-  sop_write<F16>(sop + 2 * SOP_TILE, ddpv, lane);
+// The producers run the pass 3 stream with the roles of the two sides exchanged (produce_q<KSIDE = true>): a lane
+// owns a staged query, its registers run over the wave's 32 keys. The operand tiles therefore hold rows = queries,
+// columns = keys, and the consumer, which contracts over the queries, reads them with transposing loads.
+// Per-lane part of the address of such a read: lane (key = lane % 32, h = lane / 32) receives, for k-step t, the queries
+// 16t + 4h + 0..3 (s = 0) and 16t + 8 + 4h + 0..3 (s = 1) at column `key`, the order tr_lane_off_acc gives the
+// staged Q-side tiles. Within a 16-lane group lane i addresses query row (i >> 2) and the four keys 4 (i & 3) .. + 3,
+// which the tile keeps in chunk 2b + (cg & 1), half cg >> 1 (b = key / 16, cg = i & 3).
+__device__ __forceinline__ int sop_tr_lane_off(int s, int lane) {
+  const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5, cg = i & 3;
+  const int r = 8 * s + 4 * h + (i >> 2);
+  return r * 64 + (((2 * b + (cg & 1)) ^ ((r >> 2) & 3)) << 4) + 8 * (cg >> 1);
 }
 
 template <bool F16, int D, int MASK>
@@ -387,6 +338,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kr, h);
     load_resident<D>(ddVb, (const __bf16*)p.ddv + koff, p.stride_kn, kr, h);
     const float c_scale_log2 = p.scale * kLog2e;
+    const StreamKeys<MASK> kgeo(p.mask_off, p.window, p.n_k);
     __syncthreads();
     int sp = 0;  // ring slot of tile j (slot 0 holds tile t_begin)
     for (int j = t_begin; j <= t_end; j++) {
@@ -395,9 +347,16 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
         const char* stage = smem + sp * SM::STAGE;
         char* sop = sop_base + (j & 1) * SM::SOP_BUF;
         const bool masked = geo.partial(qb, kw);
-        int lo = 0, hi = 0;  // query row 8g + 4h + e of the tile counts iff lo <= 8g + e <= hi: it exists and sees key kj
-        if (masked) keep_branch(), geo.limits(qb, kj, h, lo, hi);
-        produce_k<F16, D>(stage, sop, Kb, ddKb, Vb, ddVb, lane, lo, hi, masked, c_scale_log2, p.scale);
+        const int qi = qb + n;   // the lane's query
+        int lo = 0, hi = 0;      // key kw + 8g + 4h + e counts for it iff lo <= 8g + e <= hi
+        if (masked) {
+          keep_branch();
+          kgeo.limits(kw, qi, h, lo, hi);
+          if (qi >= p.n_q) hi = -2 * TS;   // a row past the end of the tensor (a copy of its last row)
+        }
+        const float* stat = reinterpret_cast<const float*>(stage + 3 * SM::TILE);
+        produce_q<F16, D, true>(stage, sop, Kb, ddKb, Vb, ddVb, lane, lo, hi, masked, c_scale_log2, stat[n], p.scale,
+                                stat[TS + n], stat[2 * TS + n], stat[3 * TS + n]);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
@@ -419,6 +378,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
       troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
     }
+    const int sopoff[2] = {sop_tr_lane_off(0, lane), sop_tr_lane_off(1, lane)};
     Dma<D> dma;
     dma.init(p.stride_qn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
@@ -462,7 +422,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int x = 0; x < 3; x++) a_op[t][x] = sop_read(sop + x * SOP_TILE, t, lane);
+          for (int x = 0; x < 3; x++) a_op[t][x] = lds_read_tr_pre(sop + sopoff[0], sop + sopoff[1], x * SOP_TILE + t * 16 * 64);
         bf16x8_t bop[2][3];
         bop[0][0] = lds_read_tr_pre(bp[0][0], bp[0][1], 1 * SM::TILE + 0 * 16 * 2 * D);
         bop[0][1] = lds_read_tr_pre(bp[0][0], bp[0][1], 0 * SM::TILE + 0 * 16 * 2 * D);
