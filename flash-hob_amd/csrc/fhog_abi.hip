@@ -63,6 +63,8 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->d != 32 && a->d != 64 && a->d != 128) return fail(FHOG_E_SHAPE, "head dim %lld not in {32, 64, 128}", (long long)a->d);
   if (const int rc = check_mask(a->causal, a->window, a->n_q, a->n_k)) return rc;
   if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
+  if (a->ws_bytes != 0 && a->ws_bytes < (int64_t)(3 * a->batch * a->n_q * sizeof(float)))
+    return fail(FHOG_E_SHAPE, "ws_bytes %lld is below the minimum of 3 * batch * n_q floats", (long long)a->ws_bytes);
   const int vec = a->dtype == FHOG_DTYPE_FP32 ? 4 : 8;  // elements per 16 bytes
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
   if (a->stride_qn > kMaxRowStride || a->stride_kn > kMaxRowStride) return fail(FHOG_E_STRIDE, "row stride above 2^24 elements");
@@ -118,10 +120,42 @@ fhog::Params to_params(const fhog_bwdbwd_args* a) {
   p.causal = a->causal != FHOG_MASK_NONE;
   p.f16 = a->dtype == FHOG_DTYPE_FP16;
   mask_params(a->causal, a->window, a->n_q, a->n_k, &p.mask_off, &p.window);
+  p.n_split = 1;
+  p.part = nullptr;
   return p;
 }
 
-int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& p, int impl, int pass, hipStream_t s) {
+// ---- splitting the streamed side of small launches (16-bit kernels at d = 64) ---------------------------------
+// Bytes of d | dd | b, rounded up so that what follows stays 16-byte aligned.
+size_t stats_bytes(const fhog_bwdbwd_args* a) { return ((size_t)3 * a->batch * a->n_q * sizeof(float) + 15) & ~(size_t)15; }
+// fp32 partial results one split of a pass writes
+size_t split_bytes(const fhog_bwdbwd_args* a, int pass) {
+  if (pass == FHOG_PASS_DQ_DDO) return (size_t)2 * a->batch * a->n_q * a->d * sizeof(float);
+  if (pass == FHOG_PASS_DK_DV) return (size_t)2 * a->batch * a->n_k * a->d * sizeof(float);
+  return (size_t)3 * a->batch * a->n_q * sizeof(float);
+}
+// Splits a pass would like: enough workgroups for two per CU, every split keeping at least 8 streamed tiles.
+int wanted_split(const fhog_bwdbwd_args* a, int impl, int pass) {
+  if (impl != FHOG_IMPL_BF16 || a->d != 64 || pass == FHOG_PASS_D) return 1;
+  const bool kside = pass == FHOG_PASS_DK_DV;
+  const int64_t groups = ((kside ? a->n_k : a->n_q) + 127) / 128 * a->batch;
+  const int64_t streamed = ((kside ? a->n_q : a->n_k) + 31) / 32;
+  int s = 1;
+  while (groups * s < 512 && s < 16 && streamed / (2 * s) >= 8) s *= 2;
+  return s;
+}
+// ... and what of that the workspace has room for
+int granted_split(const fhog_bwdbwd_args* a, int impl, int pass) {
+  int s = wanted_split(a, impl, pass);
+  const size_t have = a->ws_bytes > 0 ? (size_t)a->ws_bytes : 0;
+  while (s > 1 && stats_bytes(a) + (size_t)s * split_bytes(a, pass) > have) s /= 2;
+  return s;
+}
+
+int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& base, int impl, int pass, hipStream_t s) {
+  fhog::Params p = base;
+  p.n_split = granted_split(a, impl, pass);
+  p.part = reinterpret_cast<float*>(reinterpret_cast<char*>(a->ws) + stats_bytes(a));
   hipError_t e;
   if (pass == FHOG_PASS_D)
     e = fhog::launch_rowdot(p, a->dtype, s);
@@ -233,6 +267,17 @@ size_t fhog_bwdbwd_args_size(void) { return sizeof(fhog_bwdbwd_args); }
 size_t fhog_bwdbwd_workspace_bytes(int64_t batch, int64_t n_q) {
   if (batch < 0 || n_q < 0) return 0;
   return (size_t)3 * (size_t)batch * (size_t)n_q * sizeof(float);
+}
+
+size_t fhog_bwdbwd_workspace_hint(const fhog_bwdbwd_args* args) {
+  if (validate(args) != FHOG_OK) return 0;
+  const int impl = select_impl(args);
+  size_t extra = 0;
+  for (int pass = FHOG_PASS_DD; pass <= FHOG_PASS_DD_B; pass++) {
+    const int s = wanted_split(args, impl, pass);
+    if (s > 1 && (size_t)s * split_bytes(args, pass) > extra) extra = (size_t)s * split_bytes(args, pass);
+  }
+  return extra ? stats_bytes(args) + extra : fhog_bwdbwd_workspace_bytes(args->batch, args->n_q);
 }
 
 int fhog_validate(const fhog_bwdbwd_args* args) { return validate(args); }

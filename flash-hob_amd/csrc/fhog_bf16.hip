@@ -26,6 +26,50 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
+// part `split` of `n` equal parts of the streamed tile range [lo, hi) (the last parts may be empty)
+__device__ __forceinline__ void split_range(int split, int n, int& lo, int& hi) {
+  const int chunk = (hi - lo + n - 1) / n;
+  lo = min(hi, lo + split * chunk);
+  hi = min(hi, lo + chunk);
+}
+
+// Finishes a statistics pass that ran split: sums the partial row sums in a fixed order.
+template <int PASS>
+__global__ void __launch_bounds__(256) combine_stats(Params p) {
+  const int64_t rows = (int64_t)p.batch * p.n_q, row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (row >= rows) return;
+  float a = 0.f, b = 0.f, c = 0.f;
+  for (int s = 0; s < p.n_split; s++) {
+    const float* ps = p.part + (int64_t)s * 3 * rows + row;
+    if (PASS != 2) a += ps[0];
+    if (PASS != 1) b += ps[rows];
+    if (PASS == 5) c += ps[2 * rows];
+  }
+  if (PASS != 2) p.ws_dd[row] = a;
+  if (PASS == 2) p.ws_b[row] = b;
+  if (PASS == 5) p.ws_b[row] = __builtin_fmaf(-a, c, b);
+}
+
+// Finishes pass 3 or 4 that ran split: out0 = scale * sum of the first partial tensor, out1 = sum of the second,
+// rounded to the tensor type. One thread per four columns of a row.
+template <bool F16, int D>
+__global__ void __launch_bounds__(256) combine_out(const float* part, int n_split, int batch, int n, int64_t stride_b,
+                                                   int64_t stride_n, uint16_t* out0, uint16_t* out1, float scale) {
+  const int64_t rows = (int64_t)batch * n, idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = idx / (D / 4);
+  const int col = (int)(idx % (D / 4)) * 4;
+  if (row >= rows) return;
+  f32x4_t a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < n_split; s++) {
+    const float* ps = part + ((int64_t)s * 2 * rows + row) * D + col;
+    a += *reinterpret_cast<const f32x4_t*>(ps);
+    b += *reinterpret_cast<const f32x4_t*>(ps + rows * D);
+  }
+  const int64_t o = (row / n) * stride_b + (row % n) * stride_n + col;
+  *reinterpret_cast<u32x2_t*>(out0 + o) = pack4<F16>(a[0] * scale, a[1] * scale, a[2] * scale, a[3] * scale);
+  *reinterpret_cast<u32x2_t*>(out1 + o) = pack4<F16>(b[0], b[1], b[2], b[3]);
+}
+
 template <bool F16, int D, int PASS, int MASK>
 __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -34,8 +78,10 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
   constexpr int STAGE = NT * TILE;
   constexpr int KK = D / 16;
 
-  int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
+  // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
+  int bh, tile, split = 0;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, MASK != MASK_NONE, bh, tile)) return;
+  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
@@ -67,7 +113,7 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
 #pragma unroll
       for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(to_f32<F16>(Ob[kk][e]), to_f32<F16>(dOb[kk][e]), dsum);
     dsum += __shfl_xor(dsum, 32);
-    if (h == 0 && qi < p.n_q) p.ws_d[row] = dsum;
+    if (h == 0 && qi < p.n_q && split == 0) p.ws_d[row] = dsum;
   }
   const float dd = (PASS == 2 || PASS == 3) ? p.ws_dd[row] : 0.f;
   const float b = PASS == 3 ? p.ws_b[row] : 0.f;
@@ -98,10 +144,12 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
   const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
   int j_begin, j_end;  // key tiles this workgroup visits
   geo.tile_range(q0, WG_ROWS, j_begin, j_end);
+  if (p.n_split > 1) split_range(split, p.n_split, j_begin, j_end);
   Dma<D> dma;
   dma.init(p.stride_kn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-  dma.template issue_all<NT>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
+  if (j_begin < j_end)
+    dma.template issue_all<NT>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
@@ -244,6 +292,22 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
     dma_wait();
     __syncthreads();
   }
+  if (PASS == 3 && p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]
+    if (qi >= p.n_q) return;
+    const int64_t rows = (int64_t)p.batch * p.n_q;
+    float* pq = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_q + qi) * D;
+    float* po = pq + rows * D;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x16_t& x = acc_dq[cb];
+        const f32x16_t& y = acc_ddo[cb];
+        *reinterpret_cast<f32x4_t*>(pq + 32 * cb + 8 * g + 4 * h) = f32x4_t{x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+        *reinterpret_cast<f32x4_t*>(po + 32 * cb + 8 * g + 4 * h) = f32x4_t{y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]};
+      }
+    return;
+  }
   if (PASS == 3) {
     if (qi >= p.n_q) return;
     uint16_t* odq = (uint16_t*)p.dq2 + qoff + (int64_t)qi * p.stride_qn;
@@ -265,6 +329,18 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
   if (PASS == 5) {
     red_dd += __shfl_xor(red_dd, 32);
     red_pdp += __shfl_xor(red_pdp, 32);
+  }
+  if (p.n_split > 1) {   // partial sums [split][dd | b | sum P dP][batch * n_q]; combine_stats finishes the pass
+    if (h == 0 && qi < p.n_q) {
+      const int64_t rows = (int64_t)p.batch * p.n_q;
+      float* ps = p.part + (int64_t)split * 3 * rows + row;
+      if (PASS == 1) ps[0] = red;
+      if (PASS == 2) ps[rows] = red;
+      if (PASS == 5) ps[0] = red_dd * p.scale, ps[rows] = red, ps[2 * rows] = red_pdp;
+    }
+    return;
+  }
+  if (PASS == 5) {
     const float dd_i = red_dd * p.scale;
     if (h == 0 && qi < p.n_q) {
       p.ws_dd[row] = dd_i;
@@ -288,8 +364,9 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   constexpr int STAT = 4 * TS * 4;         // L log2(e), d, dd, b of the 32 staged queries
   constexpr int STAGE = 3 * TILE + STAT;   // Q, ddQ, dO tiles, statistics
 
-  int bh, tile;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
+  int bh, tile, split = 0;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, bh, tile)) return;
+  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -327,6 +404,7 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
   int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
   geo.tile_range(k0, WG_ROWS, t_begin, t_end);
+  if (p.n_split > 1) split_range(split, p.n_split, t_begin, t_end);
   Dma<D> dma;
   dma.init(p.stride_qn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
@@ -339,13 +417,14 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   auto store_stat = [&](char* stage_base) {
     if (tid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * TILE)[tid] = (tid < TS) ? stat_reg * kLog2e : stat_reg;
   };
-  {
+  if (t_begin < t_end) {
     load_stat(t_begin * TS);
     const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
     dma.template issue_all<3>(ring_lds, TILE, src, adv, wave, p.n_q - t_begin * TS);
     wait_vm0();
     store_stat(smem);
   }
+  dma_wait();
   __syncthreads();
 
   for (int j = t_begin; j < t_end; j++) {
@@ -446,6 +525,21 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
     __syncthreads();
   }
   if (kj >= p.n_k) return;
+  if (p.n_split > 1) {   // fp32 partial rows [split][dK2 | dV2][batch * n_k][D]
+    const int64_t rows = (int64_t)p.batch * p.n_k;
+    float* pk = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_k + kj) * D;
+    float* pv2 = pk + rows * D;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x16_t& x = acc_dk[cb];
+        const f32x16_t& y = acc_dv[cb];
+        *reinterpret_cast<f32x4_t*>(pk + 32 * cb + 8 * g + 4 * h) = f32x4_t{x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+        *reinterpret_cast<f32x4_t*>(pv2 + 32 * cb + 8 * g + 4 * h) = f32x4_t{y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]};
+      }
+    return;
+  }
   uint16_t* odk = (uint16_t*)p.dk2 + koff + (int64_t)kj * p.stride_kn;
   uint16_t* odv = (uint16_t*)p.dv2 + koff + (int64_t)kj * p.stride_kn;
 #pragma unroll
@@ -460,48 +554,58 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
     }
 }
 
+template <typename K>
+hipError_t launch_sweep(K kernel, unsigned grid, int smem, hipStream_t s, const Params& p) {
+  const hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, s, p);
+  return hipGetLastError();
+}
+
 template <bool F16, int D, int MASK>
 hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
-  const dim3 block(256);
-  const dim3 grid(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch));
-  const int tile = TS * 2 * D;
+  const int tile = TS * 2 * D, slices = p.batch * p.n_split;
+  const unsigned gq = grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, slices);
+  const unsigned gk = grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, slices);
+  const bool split = p.n_split > 1;
+  const int64_t rows_q = (int64_t)p.batch * p.n_q, rows_k = (int64_t)p.batch * p.n_k;
   hipError_t e;
-  if (pass == FHOG_PASS_DD) {
-    const int smem = 2 * 2 * tile;
-    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 1, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 1, MASK>), grid, block, smem, s, p);
-  } else if (pass == FHOG_PASS_DK_DV) {
-    if constexpr (D == 64) {
-      const int smem = 2 * (3 * tile + 4 * TS * 4);
-      const dim3 gk(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch));
-      e = hipFuncSetAttribute((const void*)k_sweep_bf16<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-      if (e != hipSuccess) return e;
-      hipLaunchKernelGGL((k_sweep_bf16<F16, D, MASK>), gk, block, smem, s, p);
-    } else {
-      return hipErrorInvalidValue;
-    }
-  } else if (pass == FHOG_PASS_DQ_DDO) {
-    if constexpr (D == 64) {
-      const int smem = 2 * 4 * tile;
-      e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 3, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-      if (e != hipSuccess) return e;
-      hipLaunchKernelGGL((q_sweep_bf16<F16, D, 3, MASK>), grid, block, smem, s, p);
-    } else {
-      return hipErrorInvalidValue;
-    }
-  } else if (pass == FHOG_PASS_B) {
-    const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 2, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 2, MASK>), grid, block, smem, s, p);
-  } else {
-    const int smem = 2 * 4 * tile;
-    e = hipFuncSetAttribute((const void*)q_sweep_bf16<F16, D, 5, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep_bf16<F16, D, 5, MASK>), grid, block, smem, s, p);
+  switch (pass) {
+    case FHOG_PASS_DD:
+      e = launch_sweep(q_sweep_bf16<F16, D, 1, MASK>, gq, 2 * 2 * tile, s, p);
+      if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<1>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
+      break;
+    case FHOG_PASS_B:
+      e = launch_sweep(q_sweep_bf16<F16, D, 2, MASK>, gq, 2 * 4 * tile, s, p);
+      if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<2>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
+      break;
+    case FHOG_PASS_DD_B:
+      e = launch_sweep(q_sweep_bf16<F16, D, 5, MASK>, gq, 2 * 4 * tile, s, p);
+      if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<5>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
+      break;
+    case FHOG_PASS_DQ_DDO:
+      if constexpr (D == 64) {
+        e = launch_sweep(q_sweep_bf16<F16, D, 3, MASK>, gq, 2 * 4 * tile, s, p);
+        if (e == hipSuccess && split)
+          hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_q * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
+                             p.batch, p.n_q, p.stride_qb, p.stride_qn, (uint16_t*)p.dq2, (uint16_t*)p.ddo, p.scale);
+      } else {
+        return hipErrorInvalidValue;
+      }
+      break;
+    case FHOG_PASS_DK_DV:
+      if constexpr (D == 64) {
+        e = launch_sweep(k_sweep_bf16<F16, D, MASK>, gk, 2 * (3 * tile + 4 * TS * 4), s, p);
+        if (e == hipSuccess && split)
+          hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_k * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
+                             p.batch, p.n_k, p.stride_kb, p.stride_kn, (uint16_t*)p.dk2, (uint16_t*)p.dv2, p.scale);
+      } else {
+        return hipErrorInvalidValue;
+      }
+      break;
+    default: return hipErrorInvalidValue;
   }
-  return hipGetLastError();
+  return e != hipSuccess ? e : hipGetLastError();
 }
 
 }  // namespace

@@ -42,6 +42,10 @@ struct Params {
   int32_t f16;       // 16-bit tensors are fp16 (else bf16); read by the 16-bit MFMA family only
   int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
   int32_t window;
+  // Streamed side split over n_split workgroups per stationary tile (1 = no split): each writes fp32 partial results
+  // to `part` and a combining kernel finishes the pass. Set per pass by the caller of the launchers (d = 64 kernels).
+  int32_t n_split;
+  float* part;
 };
 
 // Kernel-side view of fhog_attn_args (first-order forward and backward).

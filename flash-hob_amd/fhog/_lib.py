@@ -16,7 +16,7 @@ DTYPE_BF16, DTYPE_FP32, DTYPE_FP16 = 0, 1, 2
 IMPL_AUTO, IMPL_FP32, IMPL_BF16 = 0, 1, 2
 MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT = 0, 1, 2
 PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 ERROR_NAMES = {
     -1: "FHOG_E_NULL", -2: "FHOG_E_SHAPE", -3: "FHOG_E_DTYPE", -4: "FHOG_E_STRIDE", -5: "FHOG_E_ALIGN",
@@ -33,7 +33,7 @@ class BwdBwdArgs(Structure):
         ("batch", c_int64), ("n_q", c_int64), ("n_k", c_int64), ("d", c_int64),
         ("stride_qb", c_int64), ("stride_qn", c_int64), ("stride_kb", c_int64), ("stride_kn", c_int64),
         ("scale", c_float), ("dtype", c_int32), ("causal", c_int32), ("impl", c_int32), ("schedule", c_int32),
-        ("window", c_int64),
+        ("window", c_int64), ("ws_bytes", c_int64),
     ]
 
 
@@ -71,6 +71,8 @@ def lib() -> ctypes.CDLL:
     L.fhog_abi_version.argtypes = []
     L.fhog_bwdbwd_workspace_bytes.restype = c_size_t
     L.fhog_bwdbwd_workspace_bytes.argtypes = [c_int64, c_int64]
+    L.fhog_bwdbwd_workspace_hint.restype = c_size_t
+    L.fhog_bwdbwd_workspace_hint.argtypes = [POINTER(BwdBwdArgs)]
     L.fhog_validate.restype = c_int
     L.fhog_validate.argtypes = [POINTER(BwdBwdArgs)]
     L.fhog_select_impl.restype = c_int

@@ -71,14 +71,28 @@ def mask_code(causal, window, n_q: int, n_k: int):
     return code, int(window)
 
 
+def _workspace(args: "_lib.BwdBwdArgs", device, split: bool) -> torch.Tensor:
+    """Allocate the workspace of a call and enter it into ``args``: the three row statistics ``d | dd | b`` and, with
+    ``split``, room for the partial results of launches that split their streamed side (``fhog_bwdbwd_workspace_hint``)."""
+    batch, n_q = args.batch, args.n_q
+    nbytes = 3 * batch * n_q * 4
+    if split:
+        args.ws, args.ws_bytes = args.q, 0      # any valid pointer: the hint is computed on the host
+        nbytes = max(nbytes, int(_lib.lib().fhog_bwdbwd_workspace_hint(ctypes.byref(args))))
+    ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
+    args.ws, args.ws_bytes = ws.data_ptr(), nbytes
+    return ws
+
+
 def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, fused_stats=False,
                 window=None) -> _lib.BwdBwdArgs:
+    """``ws``: a workspace tensor of the minimum size, or None when :func:`_workspace` fills it in afterwards."""
     a = _lib.BwdBwdArgs()
     a.q, a.k, a.v, a.o, a.dO = Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dO.data_ptr()
     a.ddq, a.ddk, a.ddv = ddQ.data_ptr(), ddK.data_ptr(), ddV.data_ptr()
     a.lse = L.data_ptr()
     a.dq2, a.dk2, a.dv2, a.ddo = (t.data_ptr() for t in outs)
-    a.ws = ws.data_ptr()
+    a.ws = ws.data_ptr() if ws is not None else 0
     a.batch, a.n_q, a.d = Q.shape
     a.n_k = K.shape[1]
     a.stride_qb, a.stride_qn = Q.stride(0), Q.stride(1)
@@ -92,7 +106,8 @@ def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws,
 
 
 def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window: Optional[int] = None,
-                 impl: Optional[str] = None, fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None):
+                 impl: Optional[str] = None, fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None,
+                 split: bool = True):
     """Flash Higher-Order-Gradients: VJP of the attention backward pass.
 
     Same positional signature and return order as the reference
@@ -121,6 +136,9 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
             default schedule's value only by fp32 summation order.
         return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
         only_pass: run a single pass (0..5, see fhog._lib.PASS_*) instead of the whole chain; for tests and profiling.
+        split: allocate the larger workspace that lets launches too small to fill the GPU split their streamed side over
+            several workgroups (fp32 partial results, added in a fixed order by a second kernel); False keeps the
+            minimum workspace of three row statistics.
 
     Returns:
         dQ2, dK2, dV2, ddO shaped and typed like Q, K, V, O (+ ``(d, dd, b)`` if ``return_stats``).
@@ -171,9 +189,9 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
         ddo = torch.empty_strided(q3.shape, q3.stride(), dtype=Q.dtype, device=Q.device)
         dk2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
         dv2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
-        ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
         args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl],
-                           (dq2, dk2, dv2, ddo), ws, fused_stats, window)
+                           (dq2, dk2, dv2, ddo), None, fused_stats, window)
+        ws = _workspace(args, Q.device, split)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         L_ = _lib.lib()
         if only_pass is None:
@@ -185,7 +203,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
            dv2.view(out_shape_k) if dv2.is_contiguous() else dv2.reshape(out_shape_k),
            ddo.view(out_shape_q) if ddo.is_contiguous() else ddo.reshape(out_shape_q))
     if return_stats:
-        st = ws.view(3, *L.shape)
+        st = ws[:3 * batch * n_q].view(3, *L.shape)
         return res + ((st[0], st[1], st[2]),)
     return res
 
@@ -197,7 +215,7 @@ class BwdBwdPlan:
     """
 
     def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window=None, impl=None,
-                 fused_stats=False):
+                 fused_stats=False, split=True):
         ts = [_flatten(t, "tensor") for t in (Q, K, V, O, dO, ddQ, ddK, ddV)]
         q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = ts
         q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
@@ -206,8 +224,10 @@ class BwdBwdPlan:
         lse = L.reshape(batch, n_q).to(torch.float32).contiguous()
         self.keep = (q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse)
         self.outs = (torch.empty_like(q3), torch.empty_like(k3), torch.empty_like(v3), torch.empty_like(q3))
-        self.ws = torch.empty(3 * batch * n_q, dtype=torch.float32, device=Q.device)
-        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, self.ws, fused_stats, window)
+        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, None, fused_stats, window)
+        with torch.cuda.device(Q.device):
+            self.ws_all = _workspace(self.args, Q.device, split)   # d | dd | b, then partial results of split launches
+        self.ws = self.ws_all[:3 * batch * n_q]
         self.lib = _lib.lib()
         _lib.check(self.lib.fhog_validate(ctypes.byref(self.args)))
         self.impl = self.lib.fhog_select_impl(ctypes.byref(self.args))

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FHOG_ABI_VERSION 2
+#define FHOG_ABI_VERSION 3
 
 /* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
 #define FHOG_DTYPE_BF16 0
@@ -94,7 +94,8 @@ typedef struct fhog_bwdbwd_args {
   void* dk2; /* like k */
   void* dv2; /* like k */
   void* ddo; /* like q */
-  /* workspace: 3 * batch * n_q floats, laid out d | dd | b, each (batch, n_q) contiguous */
+  /* workspace: at least 3 * batch * n_q floats, laid out d | dd | b, each (batch, n_q) contiguous; whatever follows
+     (see ws_bytes) holds partial results of launches whose streamed side is split */
   float* ws;
   int64_t batch, n_q, n_k, d;
   /* element strides. The q group (q, o, dO, ddq, dq2, ddo) shares stride_qb/stride_qn,
@@ -106,6 +107,11 @@ typedef struct fhog_bwdbwd_args {
   int32_t impl;   /* FHOG_IMPL_* */
   int32_t schedule; /* FHOG_SCHEDULE_* */
   int64_t window; /* sliding window length in keys, 0 = none; needs a causal mask */
+  int64_t ws_bytes; /* size of ws in bytes; 0 = the minimum, fhog_bwdbwd_workspace_bytes(batch, n_q). With
+                       fhog_bwdbwd_workspace_hint(args) bytes, launches too small to fill the GPU (few batch*head
+                       slices, short sequences; d = 64 kernels) split the streamed side over several workgroups,
+                       which write fp32 partial results behind d | dd | b; a second kernel adds them in a fixed
+                       order (no atomics). Anything in between gives as much of that as fits. */
 } fhog_bwdbwd_args;
 
 /* Version of this header the library was built from. */
@@ -117,6 +123,11 @@ size_t fhog_bwdbwd_args_size(void);
 /* Bytes of workspace fhog_bwdbwd needs: 3 * batch * n_q * sizeof(float).
    Replaces the torch allocations of D, dD, B at fhog/triton_bwdbwd.py:580-584. */
 size_t fhog_bwdbwd_workspace_bytes(int64_t batch, int64_t n_q);
+
+/* Workspace size that lets every pass of these arguments use the split it would like (>= the minimum, and equal to
+   it when no pass would split); 0 if the arguments are not valid. Host-only. No counterpart in the reference, whose
+   kernels are always tiled over (batch*head, N / BLOCK) alone (fhog/triton_bwdbwd.py:586-646). */
+size_t fhog_bwdbwd_workspace_hint(const fhog_bwdbwd_args* args);
 
 /* Host-only argument check (no HIP call is made; works without a GPU).
    Returns FHOG_OK or the FHOG_E_* code fhog_bwdbwd would return for these arguments. */

@@ -34,7 +34,7 @@ def test_header_symbols_exported(L):
     assert set(names) >= {"fhog_abi_version", "fhog_bwdbwd_args_size", "fhog_bwdbwd_workspace_bytes", "fhog_validate", "fhog_select_impl",
                           "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error",
                           "fhog_attn_args_size", "fhog_attn_validate", "fhog_attn_fwd", "fhog_attn_bwd",
-                          "fhog_probe_mfma_rate"}
+                          "fhog_probe_mfma_rate", "fhog_bwdbwd_workspace_hint"}
     for n in names:
         assert hasattr(L, n), n
 
@@ -56,7 +56,7 @@ def _header_fields(struct_name):
 def test_struct_mirror_matches_header():
     from fhog import _lib
     assert _header_fields("fhog_bwdbwd_args") == [f[0] for f in _lib.BwdBwdArgs._fields_]
-    assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 208
+    assert ctypes.sizeof(_lib.BwdBwdArgs) == _lib.lib().fhog_bwdbwd_args_size() == 216
     assert _header_fields("fhog_attn_args") == [f[0] for f in _lib.AttnArgs._fields_]
     assert ctypes.sizeof(_lib.AttnArgs) == _lib.lib().fhog_attn_args_size() == 160
 
@@ -101,7 +101,7 @@ def test_attn_validate(L, mutate, backward, code, word):
 
 
 def test_version_and_workspace(L):
-    assert L.fhog_abi_version() == 2
+    assert L.fhog_abi_version() == 3
     assert L.fhog_bwdbwd_workspace_bytes(32, 4096) == 3 * 32 * 4096 * 4
     assert L.fhog_bwdbwd_workspace_bytes(-1, 5) == 0
 
@@ -135,6 +135,7 @@ def test_validate_accepts_good(L):
     (lambda a: setattr(a, "window", 16), -6, "window needs"),
     (lambda a: (setattr(a, "causal", 2), setattr(a, "window", -1)), -6, "window"),
     (lambda a: setattr(a, "scale", float("nan")), -9, "scale"),
+    (lambda a: setattr(a, "ws_bytes", 3 * 4 * 256 * 4 - 4), -2, "ws_bytes"),
 ])
 def test_validate_rejects(L, mutate, code, word):
     a = good_args()
@@ -144,6 +145,27 @@ def test_validate_rejects(L, mutate, code, word):
     # the compute entry points refuse the same way, before any launch
     assert L.fhog_bwdbwd(ctypes.byref(a), None) == code
     assert L.fhog_bwdbwd_pass(ctypes.byref(a), 1, None) == code
+
+
+def test_workspace_hint(L):
+    """The hint is the minimum where no pass would split, and grows by the partial results of the widest split
+    where the launch is too small to fill the GPU (16-bit kernels at d = 64 only)."""
+    a = good_args()                           # bf16, batch 4, 256 x 512, d = 64: 8 workgroups of 128 rows
+    minimum = L.fhog_bwdbwd_workspace_bytes(4, 256)
+    assert minimum == 3 * 4 * 256 * 4
+    # 16 key tiles: one split in two keeps 8 tiles each -> pass 3 wants 2 x (2 * batch * n_q * d) floats
+    assert L.fhog_bwdbwd_workspace_hint(ctypes.byref(a)) == minimum + 2 * (2 * 4 * 256 * 64 * 4)
+    a.ws_bytes = minimum
+    assert L.fhog_validate(ctypes.byref(a)) == 0
+    a.ws_bytes = 0
+    a.batch = 4096                            # plenty of workgroups: nothing to split
+    a.stride_qb, a.stride_kb = 256 * 64, 512 * 64
+    assert L.fhog_bwdbwd_workspace_hint(ctypes.byref(a)) == L.fhog_bwdbwd_workspace_bytes(4096, 256)
+    a = good_args()
+    a.dtype = 1                               # fp32 tensors: the fp32-MFMA family does not split
+    assert L.fhog_bwdbwd_workspace_hint(ctypes.byref(a)) == minimum
+    a.d = 96
+    assert L.fhog_bwdbwd_workspace_hint(ctypes.byref(a)) == 0   # invalid arguments
 
 
 def test_probe_rejects_bad_arguments(L):

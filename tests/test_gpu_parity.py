@@ -246,6 +246,39 @@ def test_bf16_chain_writes_row_sums_d_itself(shape, dtype, fused_stats):
     assert normalised_max_error(plan.ws.view(3, -1)[0], got) < 1e-5
 
 
+@pytest.mark.parametrize("fused_stats", [False, True])
+@pytest.mark.parametrize("case", [((1, 2048, 2048, 64), False, None, torch.bfloat16), ((1, 2048, 2048, 64), True, None, torch.float16),
+                                  ((2, 1000, 1500, 64), "bottom_right", None, torch.bfloat16),
+                                  ((1, 1536, 1536, 64), True, 300, torch.bfloat16), ((1, 130, 4100, 64), False, None, torch.bfloat16)])
+def test_split_streamed_side_matches_the_unsplit_launch(case, fused_stats):
+    """Few (batch*head) slices at d = 64: with the workspace of fhog_bwdbwd_workspace_hint every pass splits its
+    streamed side over several workgroups (fp32 partial results, added by a second kernel). Same gate against the
+    fp64 oracle as the unsplit launch, row statistics equal up to summation order, outputs within a 16-bit rounding."""
+    from fhog import BwdBwdPlan, _lib
+    (batch, n_q, n_k, d), causal, window, dtype = case
+    scale = d ** -0.5
+    x = with_caches(make_case(batch, n_q, n_k, d, dtype, seed=23, grad_std=0.1), scale, causal, window)
+    plans = [BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], scale, causal=causal,
+                        window=window, impl="bf16", fused_stats=fused_stats, split=sp) for sp in (True, False)]
+    assert plans[0].args.ws_bytes > plans[1].args.ws_bytes == _lib.lib().fhog_bwdbwd_workspace_bytes(batch, n_q)
+    res = []
+    for plan in plans:
+        plan.ws_all.fill_(float("nan"))
+        outs = [o.clone() for o in plan.run()]
+        torch.cuda.synchronize()
+        assert torch.isfinite(plan.ws).all()
+        res.append((outs, plan.ws.clone().view(3, -1)))
+    ref = reference_fp64_cpu(x, scale, causal, window)
+    order = ("dq2", "dk2", "dv2", "ddo")   # the plan's output order
+    for outs, _ in res:
+        e = {n: normalised_max_error(o.view_as(x["Q"] if n in ("dq2", "ddo") else x["K"]), ref[n]) for n, o in zip(order, outs)}
+        assert max(e.values()) < 2e-2, e
+    for a, b in zip(res[0][1], res[1][1]):
+        assert normalised_max_error(a, b) < 1e-5
+    for a, b in zip(res[0][0], res[1][0]):
+        assert normalised_max_error(a, b) < 1e-2
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("impl", ["bf16", "fp32"])
 @pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
