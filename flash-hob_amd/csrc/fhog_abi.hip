@@ -125,7 +125,7 @@ fhog::Params to_params(const fhog_bwdbwd_args* a) {
   return p;
 }
 
-// ---- splitting the streamed side of small launches (16-bit kernels at d = 64) ---------------------------------
+// ---- splitting the streamed side of small launches (16-bit kernels) -------------------------------------------
 // Bytes of d | dd | b, rounded up so that what follows stays 16-byte aligned.
 size_t stats_bytes(const fhog_bwdbwd_args* a) { return ((size_t)3 * a->batch * a->n_q * sizeof(float) + 15) & ~(size_t)15; }
 // fp32 partial results one split of a pass writes
@@ -136,7 +136,7 @@ size_t split_bytes(const fhog_bwdbwd_args* a, int pass) {
 }
 // Splits a pass would like: enough workgroups for two per CU, every split keeping at least 8 streamed tiles.
 int wanted_split(const fhog_bwdbwd_args* a, int impl, int pass) {
-  if (impl != FHOG_IMPL_BF16 || a->d != 64 || pass == FHOG_PASS_D) return 1;
+  if (impl != FHOG_IMPL_BF16 || pass == FHOG_PASS_D) return 1;
   const bool kside = pass == FHOG_PASS_DK_DV;
   const int64_t groups = ((kside ? a->n_k : a->n_q) + 127) / 128 * a->batch;
   const int64_t streamed = ((kside ? a->n_q : a->n_k) + 31) / 32;

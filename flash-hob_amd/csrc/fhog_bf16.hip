@@ -26,13 +26,6 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-// part `split` of `n` equal parts of the streamed tile range [lo, hi) (the last parts may be empty)
-__device__ __forceinline__ void split_range(int split, int n, int& lo, int& hi) {
-  const int chunk = (hi - lo + n - 1) / n;
-  lo = min(hi, lo + split * chunk);
-  hi = min(hi, lo + chunk);
-}
-
 // Finishes a statistics pass that ran split: sums the partial row sums in a fixed order.
 template <int PASS>
 __global__ void __launch_bounds__(256) combine_stats(Params p) {
@@ -620,7 +613,19 @@ bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
   // d = 128: passes 3 and 4 need the producer/consumer split to fit the registers; d = 64: single-role kernels throughout
-  if (p.d == 128 && (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV)) return launch_bf16_pc_pass(p, pass, s);
+  if (p.d == 128 && (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV)) {
+    const hipError_t e = launch_bf16_pc_pass(p, pass, s);
+    if (e != hipSuccess || p.n_split == 1) return e;
+    const bool kside = pass == FHOG_PASS_DK_DV;
+    const int n = kside ? p.n_k : p.n_q;
+    const dim3 grid((unsigned)(((int64_t)p.batch * n * (128 / 4) + 255) / 256));
+    uint16_t* out0 = (uint16_t*)(kside ? p.dk2 : p.dq2);
+    uint16_t* out1 = (uint16_t*)(kside ? p.dv2 : p.ddo);
+    const int64_t sb = kside ? p.stride_kb : p.stride_qb, sn = kside ? p.stride_kn : p.stride_qn;
+    if (p.f16) hipLaunchKernelGGL((combine_out<true, 128>), grid, dim3(256), 0, s, p.part, p.n_split, p.batch, n, sb, sn, out0, out1, p.scale);
+    else hipLaunchKernelGGL((combine_out<false, 128>), grid, dim3(256), 0, s, p.part, p.n_split, p.batch, n, sb, sn, out0, out1, p.scale);
+    return hipGetLastError();
+  }
   if (pass < FHOG_PASS_DD || pass > FHOG_PASS_DD_B) return hipErrorInvalidValue;
   const int mask = mask_mode(p);
 #define FHOG_SINGLE(F, DD)                                                             \

@@ -140,8 +140,10 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   using SM = PCSmem<D, false>;
   constexpr int NC = D / 32;
 
-  int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, bh, tile)) return;
+  // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
+  int bh, tile, split = 0;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, MASK != MASK_NONE, bh, tile)) return;
+  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
@@ -152,6 +154,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
   int j_begin, j_end;  // key tiles this workgroup visits
   geo.tile_range(q0, WG_ROWS, j_begin, j_end);
+  if (p.n_split > 1) split_range(split, p.n_split, j_begin, j_end);
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
@@ -205,7 +208,8 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
     Dma<D> dma;
     dma.init(p.stride_kn, wq, lane);
     const uint32_t ring_lds = lds_addr(smem);
-    dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
+    if (j_begin < j_end)
+      dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
     dma_wait();
     __syncthreads();
     int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
@@ -278,6 +282,24 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
     // acc[qb][cl][r] holds (query qw0 + 32 qb + 8*(r/4) + 4h + r%4, column 32*(NCL*ch + cl) + n)
+    if (p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]; combine_out finishes the pass
+      const int64_t rows = (int64_t)p.batch * p.n_q;
+      float* pq = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_q) * D;
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int cl = 0; cl < NCL; cl++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
+            if (qrow < p.n_q) {
+              const int64_t o = (int64_t)qrow * D + 32 * (NCL * ch + cl) + n;
+              pq[o] = acc_dq[qb][cl][r];
+              pq[rows * D + o] = acc_ddo[qb][cl][r];
+            }
+          }
+      return;
+    }
     uint16_t* odq = (uint16_t*)p.dq2 + qoff;
     uint16_t* oddo = (uint16_t*)p.ddo + qoff;
 #pragma unroll
@@ -316,8 +338,9 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   using SM = PCSmem<D, true>;
   constexpr int NC = D / 32;
 
-  int bh, tile;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
+  int bh, tile, split = 0;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, bh, tile)) return;
+  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const bool producer = wave < 4;
@@ -329,6 +352,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
   int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
   geo.tile_range(k0, WG_ROWS, t_begin, t_end);
+  if (p.n_split > 1) split_range(split, p.n_split, t_begin, t_end);
   char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
 
   if (producer) {
@@ -393,7 +417,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     auto store_stat = [&](char* stage_base) {
       if (ctid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * SM::TILE)[ctid] = (ctid < TS) ? stat_reg * kLog2e : stat_reg;
     };
-    {
+    if (t_begin < t_end) {
       const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
       dma.template issue_all<3>(ring_lds, SM::TILE, src, adv, wq, p.n_q - t_begin * TS);
       load_stat(t_begin * TS);
@@ -449,6 +473,22 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       sc = (sc == RING - 1) ? 0 : sc + 1;
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
+    if (p.n_split > 1) {   // fp32 partial rows [split][dK2 | dV2][batch * n_k][D]
+      const int64_t rows = (int64_t)p.batch * p.n_k;
+      float* pk = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_k) * D;
+#pragma unroll
+      for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int krow = kw + 8 * (r / 4) + 4 * h + (r % 4);
+          if (krow < p.n_k) {
+            const int64_t o = (int64_t)krow * D + cb * 32 + n;
+            pk[o] = acc_dk[cb][r];
+            pk[rows * D + o] = acc_dv[cb][r];
+          }
+        }
+      return;
+    }
     uint16_t* odk = (uint16_t*)p.dk2 + koff;
     uint16_t* odv = (uint16_t*)p.dv2 + koff;
 #pragma unroll
@@ -473,12 +513,12 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
     const int smem = PCSmem<D, false>::TOTAL;
     e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((q_sweep3_pc<F16, D, MASK>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((q_sweep3_pc<F16, D, MASK>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split)), block, smem, s, p);
   } else {
     const int smem = PCSmem<D, true>::TOTAL;
     e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_sweep_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
+    hipLaunchKernelGGL((k_sweep_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split)), block, smem, s, p);
   }
   return hipGetLastError();
 }

@@ -266,6 +266,12 @@ struct StreamQueries {
     hi = min(MASK == MASK_BAND ? j - off + win - 1 - t0 : TS, n_q - 1 - t0) - 4 * h;
   }
 };
+// part `split` of `n` equal parts of the streamed tile range [lo, hi) (the last parts may be empty)
+__device__ __forceinline__ void split_range(int split, int n, int& lo, int& hi) {
+  const int chunk = (hi - lo + n - 1) / n;
+  lo = min(hi, lo + split * chunk);
+  hi = min(hi, lo + chunk);
+}
 // mask mode of a launch (Params or AttnParams)
 template <typename P>
 inline int mask_mode(const P& p) {

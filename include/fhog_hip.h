@@ -109,7 +109,7 @@ typedef struct fhog_bwdbwd_args {
   int64_t window; /* sliding window length in keys, 0 = none; needs a causal mask */
   int64_t ws_bytes; /* size of ws in bytes; 0 = the minimum, fhog_bwdbwd_workspace_bytes(batch, n_q). With
                        fhog_bwdbwd_workspace_hint(args) bytes, launches too small to fill the GPU (few batch*head
-                       slices, short sequences; d = 64 kernels) split the streamed side over several workgroups,
+                       slices, short sequences; 16-bit kernels) split the streamed side over several workgroups,
                        which write fp32 partial results behind d | dd | b; a second kernel adds them in a fixed
                        order (no atomics). Anything in between gives as much of that as fits. */
 } fhog_bwdbwd_args;

@@ -249,9 +249,11 @@ def test_bf16_chain_writes_row_sums_d_itself(shape, dtype, fused_stats):
 @pytest.mark.parametrize("fused_stats", [False, True])
 @pytest.mark.parametrize("case", [((1, 2048, 2048, 64), False, None, torch.bfloat16), ((1, 2048, 2048, 64), True, None, torch.float16),
                                   ((2, 1000, 1500, 64), "bottom_right", None, torch.bfloat16),
-                                  ((1, 1536, 1536, 64), True, 300, torch.bfloat16), ((1, 130, 4100, 64), False, None, torch.bfloat16)])
+                                  ((1, 1536, 1536, 64), True, 300, torch.bfloat16), ((1, 130, 4100, 64), False, None, torch.bfloat16),
+                                  ((1, 2048, 2048, 128), True, None, torch.bfloat16), ((2, 1000, 1500, 128), False, None, torch.float16),
+                                  ((1, 1536, 1536, 128), "bottom_right", 700, torch.bfloat16)])
 def test_split_streamed_side_matches_the_unsplit_launch(case, fused_stats):
-    """Few (batch*head) slices at d = 64: with the workspace of fhog_bwdbwd_workspace_hint every pass splits its
+    """Few (batch*head) slices: with the workspace of fhog_bwdbwd_workspace_hint every pass splits its
     streamed side over several workgroups (fp32 partial results, added by a second kernel). Same gate against the
     fp64 oracle as the unsplit launch, row statistics equal up to summation order, outputs within a 16-bit rounding."""
     from fhog import BwdBwdPlan, _lib
@@ -334,7 +336,9 @@ def test_bf16_family_ragged_lengths(shape, causal, fused_stats):
     plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], scale, causal=causal,
                       impl="bf16", fused_stats=fused_stats)
     big = [torch.full((t.numel() + 4096,), canary, dtype=t.dtype, device=t.device) for t in plan.outs]
-    ws_big = torch.full((plan.ws.numel() + 1024,), canary, dtype=torch.float32, device="cuda")
+    ws_floats = (plan.args.ws_bytes + 3) // 4   # d | dd | b and, for a split launch, the partial results
+    assert ws_floats <= plan.ws_all.numel()
+    ws_big = torch.full((ws_floats + 1024,), canary, dtype=torch.float32, device="cuda")
     for name, buf, t in zip(("dq2", "dk2", "dv2", "ddo"), big, plan.outs):
         setattr(plan.args, name, buf.data_ptr())
     plan.args.ws = ws_big.data_ptr()
@@ -343,7 +347,7 @@ def test_bf16_family_ragged_lengths(shape, causal, fused_stats):
     for buf, t, o in zip(big, plan.outs, outs[:4]):
         assert torch.equal(buf[:t.numel()].view(t.shape), o.reshape(t.shape))
         assert (buf[t.numel():] == canary).all()
-    assert (ws_big[plan.ws.numel():] == canary).all()
+    assert (ws_big[ws_floats:] == canary).all()
 
 
 def test_bf16_auto_dispatch():
@@ -438,20 +442,28 @@ def test_headline_properties_linearity_zero_and_sdpa_case():
 
 
 def test_peak_memory_is_linear_in_n():
-    """Workspace + outputs only: 4 output tensors and 3 fp32 row vectors, nothing of size N_Q x N_K."""
+    """Workspace + outputs only: 4 output tensors and 3 fp32 row vectors, nothing of size N_Q x N_K. The larger
+    workspace for split launches adds partial results of at most 2 * 65536 * d floats, whatever N (the number of
+    splits falls as the number of workgroups grows)."""
     import fhog
     sizes = {}
     for n in (2048, 8192):
         x = with_caches(make_case(4, n, n, 128, torch.bfloat16, seed=7, grad_std=0.1), 128 ** -0.5, True)
-        torch.cuda.synchronize()
-        torch.cuda.reset_peak_memory_stats()
-        before = torch.cuda.memory_allocated()
-        outs = run_fhog(x, 128 ** -0.5, True)
-        torch.cuda.synchronize()
-        sizes[n] = torch.cuda.max_memory_allocated() - before
-        expect = 4 * 4 * n * 128 * 2 + 3 * 4 * n * 4
-        assert sizes[n] <= expect * 1.05 + (1 << 20), (n, sizes[n], expect)
-        del outs, x
+        for split in (False, True):
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            before = torch.cuda.memory_allocated()
+            outs = run_fhog(x, 128 ** -0.5, True, split=split)
+            torch.cuda.synchronize()
+            used = torch.cuda.max_memory_allocated() - before
+            expect = 4 * 4 * n * 128 * 2 + 3 * 4 * n * 4
+            if split:
+                assert used <= expect * 1.05 + (1 << 20) + 2 * 65536 * 128 * 4, (n, used, expect)
+            else:
+                sizes[n] = used
+                assert used <= expect * 1.05 + (1 << 20), (n, used, expect)
+            del outs
+        del x
     assert sizes[8192] <= 4.2 * sizes[2048]
 
 
