@@ -411,6 +411,7 @@ hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
 // which: 0 forward, 1 backward Q-tiled (dQ), 2 backward K-tiled (dK, dV)
 hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
+  if (which == 2 && p.d == 128) return launch_attn_bwd_k_pc(p, s);   // one wave does not hold this sweep at d = 128
   const int mask = mask_mode(p);
 #define FHOG_ATTN(F, DD)                                                            \
   (mask == MASK_NONE ? launch_attn_d<F, DD, MASK_NONE>(p, which, s)                 \

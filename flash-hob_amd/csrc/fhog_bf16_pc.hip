@@ -505,6 +505,221 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   }
 }
 
+// ---- first-order backward, K-tiled (dK, dV) at d = 128 -------------------------------------------------------------
+// The arithmetic of fhog/triton_flash.py:201-220 for one key tile, as a producer/consumer kernel of the same shape as
+// pass 4: a single wave does not hold two 32 x 128 fp32 accumulators, two resident tensors and the S-shaped tiles in 256
+// registers (the single-role kernel of fhog_attn.hip keeps 24-37 registers per lane in scratch memory at d = 128).
+//   producers: S = K Q^T, dP = V dO^T (resident operand first: a lane owns one staged query), P = exp2(S c - L),
+//              dS = P (dP - d); operand tiles dS, P
+//   consumers: dK^T += dS^T Q, dV^T += P^T dO from transposing reads of the operand and the staged tiles
+template <int D>
+struct PCSmemAttn {
+  static constexpr int NT = 2;      // streamed tensors per stage: Q, dO
+  static constexpr int NSOP = 2;    // operand tensors handed over per block: dS, P
+  static constexpr int TILE = TS * 2 * D;
+  static constexpr int STAT = 2 * TS * (int)sizeof(float);   // L log2(e), d of the 32 staged queries
+  static constexpr int STAGE = NT * TILE + STAT;
+  static constexpr int SOP_WAVE = NSOP * SOP_TILE;
+  static constexpr int SOP_BUF = 4 * SOP_WAVE;
+  static constexpr int SOP_BASE = RING * STAGE;
+  static constexpr int TOTAL = SOP_BASE + 2 * SOP_BUF;
+};
+
+template <bool F16, int D>
+__device__ __forceinline__ void produce_first(const char* stage, char* sop, const bf16x8_t* Kb, const bf16x8_t* Vb, int lane,
+                                              int lo, int hi, bool mask, float c_scale_log2, float l_log2, float dsum) {
+  constexpr int TILE = TS * 2 * D;
+  constexpr int KK = D / 16, NSTEP = 2 * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
+  const int n = lane & 31, h = lane >> 5;
+  int aoff[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+  f32x16_t s = {0}, dp = {0}, pv;
+  bf16x8_t a[NB];
+#pragma unroll
+  for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + (i / KK) * TILE, aoff[i % KK]);
+#pragma unroll
+  for (int i = 0; i < NSTEP; i++) {
+    const int ph = i / KK, kk = i % KK, c = i % NB;
+    if (i + PF < NSTEP) a[(i + PF) % NB] = lds_read128(stage + ((i + PF) / KK) * TILE, aoff[(i + PF) % KK]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ph == 0) {
+      s = mfma<F16>(Kb[kk], a[c], s);
+    } else {
+      dp = mfma<F16>(Vb[kk], a[c], dp);
+#pragma unroll
+      for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (mask) {  // wave-uniform: the block holds hidden pairs (mask edge or end of a tensor)
+    keep_branch();
+#pragma unroll
+    for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+  }
+  uint32_t pk_ds[8], pk_p[8];
+#pragma unroll
+  for (int r = 0; r < 16; r += 2) {
+    pk_ds[r / 2] = pack2<F16>(pv[r] * (dp[r] - dsum), pv[r + 1] * (dp[r + 1] - dsum));
+    pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
+  }
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+    sop_write_pk(sop + 0 * SOP_TILE, pk_ds, t, lane);
+    sop_write_pk(sop + 1 * SOP_TILE, pk_p, t, lane);
+  }
+}
+
+template <bool F16, int D, int MASK>
+__global__ void __launch_bounds__(PC_THREADS) attn_bwd_k_pc(AttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  using SM = PCSmemAttn<D>;
+  constexpr int NC = D / 32;
+
+  int bh, tile;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave < 4;
+  const int wq = wave & 3;
+  const int n = lane & 31, h = lane >> 5;
+  const int k0 = tile * WG_ROWS, kw = k0 + 32 * wq, kj = kw + n;
+  const int kr = min(kj, p.n_k - 1);  // keys past the end compute on a copy of the last row; nothing of them is stored
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const StreamQueries<MASK> geo(p.mask_off, p.window, p.n_q);
+  int t_begin, t_end;  // query tiles that hold a query seeing some key of this workgroup
+  geo.tile_range(k0, WG_ROWS, t_begin, t_end);
+  char* sop_base = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
+
+  if (producer) {
+    bf16x8_t Kb[D / 16], Vb[D / 16];
+    load_resident<D>(Kb, (const __bf16*)p.k + koff, p.stride_kn, kr, h);
+    load_resident<D>(Vb, (const __bf16*)p.v + koff, p.stride_kn, kr, h);
+    const float c_scale_log2 = p.scale * kLog2e;
+    const StreamKeys<MASK> kgeo(p.mask_off, p.window, p.n_k);
+    __syncthreads();
+    int sp = 0;  // ring slot of tile j (slot 0 holds tile t_begin)
+    for (int j = t_begin; j <= t_end; j++) {
+      const int qb = j * TS;
+      if (j < t_end && !geo.dead(qb, kw)) {
+        const char* stage = smem + sp * SM::STAGE;
+        char* sop = sop_base + (j & 1) * SM::SOP_BUF;
+        const bool masked = geo.partial(qb, kw);
+        const int qi = qb + n;   // the lane's query
+        int lo = 0, hi = 0;      // key kw + 8g + 4h + e counts for it iff lo <= 8g + e <= hi
+        if (masked) {
+          keep_branch();
+          kgeo.limits(kw, qi, h, lo, hi);
+          if (qi >= p.n_q) hi = -2 * TS;   // a row past the end of the tensor (a copy of its last row)
+        }
+        const float* stat = reinterpret_cast<const float*>(stage + SM::NT * SM::TILE);
+        produce_first<F16, D>(stage, sop, Kb, Vb, lane, lo, hi, masked, c_scale_log2, stat[n], stat[TS + n]);
+      }
+      __syncthreads();
+      sp = (sp == RING - 1) ? 0 : sp + 1;
+    }
+  } else {
+    const int ctid = tid - 256;
+    const __bf16* src[2] = {(const __bf16*)p.q + qoff, (const __bf16*)p.dO + qoff};
+    const float* stat_src = (ctid < TS ? p.lse : p.ws_d) + (int64_t)bh * p.n_q;
+    f32x16_t acc_dk[NC], acc_dv[NC];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      acc_dk[cb] = f32x16_t{0};
+      acc_dv[cb] = f32x16_t{0};
+    }
+    int troff[NC][2];
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) {
+      troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+      troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+    }
+    const int sopoff[2] = {sop_tr_lane_off(0, lane), sop_tr_lane_off(1, lane)};
+    Dma<D> dma;
+    dma.init(p.stride_qn, wq, lane);
+    const uint32_t ring_lds = lds_addr(smem);
+    float stat_reg = 0.f;  // consumer threads 0..63: one statistic value of the staged tile
+    // a global (not generic) load issued before the staging loads of the step and first touched at its end
+    auto load_stat = [&](int q_base) {
+      if (ctid < 2 * TS) stat_reg = *(global_f32_ptr)(stat_src + min(q_base + (ctid % TS), p.n_q - 1));
+    };
+    auto store_stat = [&](char* stage_base) {
+      if (ctid < 2 * TS) reinterpret_cast<float*>(stage_base + SM::NT * SM::TILE)[ctid] = (ctid < TS) ? stat_reg * kLog2e : stat_reg;
+    };
+    if (t_begin < t_end) {
+      const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
+      dma.template issue_all<2>(ring_lds, SM::TILE, src, adv, wq, p.n_q - t_begin * TS);
+      load_stat(t_begin * TS);
+      store_stat(smem);
+    }
+    dma_wait();
+    __syncthreads();
+    int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
+    for (int j = t_begin; j <= t_end; j++) {
+      if (j + 1 < t_end) {
+        const uint32_t dst = ring_lds + sn * SM::STAGE;
+        const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
+        load_stat((j + 1) * TS);
+        dma.template issue_all<2>(dst, SM::TILE, src, adv, wq, p.n_q - (j + 1) * TS);
+      }
+      if (j > t_begin && !geo.dead((j - 1) * TS, kw)) {
+        const char* stage = smem + sc * SM::STAGE;
+        const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
+        bf16x8_t a_op[2][2];   // [k-step][dS | P]
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int x = 0; x < 2; x++) a_op[t][x] = lds_read_tr_pre(sop + sopoff[0], sop + sopoff[1], x * SOP_TILE + t * 16 * 64);
+        bf16x8_t bop[2][2];    // [buffer][Q | dO]
+#pragma unroll
+        for (int x = 0; x < 2; x++) bop[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * SM::TILE);
+#pragma unroll
+        for (int it = 0; it < 2 * NC; it++) {
+          const int t = it / NC, cb = it % NC, c = it & 1;
+          if (it + 1 < 2 * NC) {
+            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+#pragma unroll
+            for (int x = 0; x < 2; x++)
+              bop[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * SM::TILE + t1 * 16 * 2 * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          acc_dk[cb] = mfma<F16>(a_op[t][0], bop[c][0], acc_dk[cb]);
+          acc_dv[cb] = mfma<F16>(a_op[t][1], bop[c][1], acc_dv[cb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (j + 1 < t_end) store_stat(smem + sn * SM::STAGE);
+      dma_wait();
+      __syncthreads();
+      sc = (sc == RING - 1) ? 0 : sc + 1;
+      sn = (sn == RING - 1) ? 0 : sn + 1;
+    }
+    // acc[cb][r] holds (key kw + 8*(r/4) + 4h + r%4, column 32 cb + n)
+    uint16_t* odk = (uint16_t*)p.dk + koff;
+    uint16_t* odv = (uint16_t*)p.dv + koff;
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int krow = kw + 8 * (r / 4) + 4 * h + (r % 4);
+        if (krow < p.n_k) {
+          const int64_t o = (int64_t)krow * p.stride_kn + cb * 32 + n;
+          odk[o] = to_elem<F16>(acc_dk[cb][r] * p.scale);
+          odv[o] = to_elem<F16>(acc_dv[cb][r]);
+        }
+      }
+  }
+}
+
+template <bool F16, int D, int MASK>
+hipError_t launch_attn_bwd_k_pc_d(const AttnParams& p, hipStream_t s) {
+  const int smem = PCSmemAttn<D>::TOTAL;
+  const hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_k_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((attn_bwd_k_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), dim3(PC_THREADS), smem, s, p);
+  return hipGetLastError();
+}
+
 template <bool F16, int D, int MASK>
 hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(PC_THREADS);
@@ -524,6 +739,17 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
 }
 
 }  // namespace
+
+// first-order backward, K-tiled, d = 128 (the other head dims run on the single-role kernel of fhog_attn.hip)
+hipError_t launch_attn_bwd_k_pc(const AttnParams& p, hipStream_t s) {
+  if (p.d != 128) return hipErrorInvalidValue;
+  const int mask = mask_mode(p);
+#define FHOG_BWDK(F)                                                                     \
+  (mask == MASK_NONE ? launch_attn_bwd_k_pc_d<F, 128, MASK_NONE>(p, s)                   \
+                     : mask == MASK_CAUSAL ? launch_attn_bwd_k_pc_d<F, 128, MASK_CAUSAL>(p, s) : launch_attn_bwd_k_pc_d<F, 128, MASK_BAND>(p, s))
+  return p.f16 ? FHOG_BWDK(true) : FHOG_BWDK(false);
+#undef FHOG_BWDK
+}
 
 hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s) {
   const int mask = mask_mode(p);
