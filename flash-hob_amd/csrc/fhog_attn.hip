@@ -262,7 +262,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
     }
 }
 
-// ---- backward, K-tiled: dK, dV ---------------------------------------------------------------------------
+// ---- backward, K-tiled: dK, dV (d = 64; at d = 128 attn_bwd_k_pc of fhog_bf16_pc.hip) ---------------------------------
 template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -402,7 +402,11 @@ hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
   switch (which) {
     case 0: return launch(attn_fwd_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
     case 1: return launch(attn_bwd_q_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    default: return launch(attn_bwd_k_bf16<F16, D, MASK>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
+    default:
+      if constexpr (D == 64)
+        return launch(attn_bwd_k_bf16<F16, D, MASK>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
+      else
+        return hipErrorInvalidValue;   // d = 128 is dispatched to the producer/consumer kernel before this point
   }
 }
 
