@@ -132,7 +132,11 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
 #pragma unroll
       for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, x[r]);
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-      const float m_new = fmaxf(m, tmax);
+      // The running maximum follows the row maximum only in jumps of more than kMaxSlack (in log2 units): P may then
+      // reach 2^kMaxSlack instead of 1, which costs no precision in a 16-bit float or in the fp32 sums, and the output
+      // accumulators are rescaled only in the rare steps where some row jumps (else on about every second tile).
+      constexpr float kMaxSlack = 8.f;
+      const float m_new = tmax > m + kMaxSlack ? tmax : m;
       // a row whose window starts in a later tile has seen no key yet: keep exp2(-inf - (-inf)) out of it
       const float m_ref = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
