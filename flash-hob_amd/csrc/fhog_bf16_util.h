@@ -100,13 +100,6 @@ __device__ __forceinline__ void sop_write_step(char* tile, u32x4_t pk, int t, in
   const int n = lane & 31, h = lane >> 5;
   *reinterpret_cast<u32x4_t*>(tile + n * 64 + (((2 * t + h) ^ ((n >> 2) & 3)) << 4)) = pk;
 }
-template <bool F16>
-__device__ __forceinline__ void sop_write(char* tile, const f32x16_t& x, int lane) {
-#pragma unroll
-  for (int t = 0; t < 2; t++)
-    sop_write_step(tile, u32x4_t{pack2<F16>(x[8 * t], x[8 * t + 1]), pack2<F16>(x[8 * t + 2], x[8 * t + 3]),
-                                 pack2<F16>(x[8 * t + 4], x[8 * t + 5]), pack2<F16>(x[8 * t + 6], x[8 * t + 7])}, t, lane);
-}
 // consumer: A operand of second-level step t: stationary row n, streamed rows in the order given above
 __device__ __forceinline__ bf16x8_t sop_read(const char* tile, int t, int lane) {
   const int n = lane & 31, h = lane >> 5;
