@@ -281,6 +281,45 @@ def test_split_streamed_side_matches_the_unsplit_launch(case, fused_stats):
         assert normalised_max_error(a, b) < 1e-2
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_split_launches_on_random_shapes_against_the_fp32_family(seed):
+    """Random ragged lengths, masks, head dims and row strides in the range where launches split (few slices, at least
+    16 streamed tiles): the 16-bit kernels with partial results against the fp32-MFMA kernels on the same tensors."""
+    import random
+    rnd = random.Random(1000 + seed)
+    d = rnd.choice([64, 128])
+    batch = rnd.choice([1, 2, 3])
+    n_q, n_k = rnd.randint(520, 2300), rnd.randint(520, 2300)
+    kind = rnd.choice(["none", "causal", "bottom_right", "band"])
+    causal, window = False, None
+    if kind == "causal":
+        causal, n_k = True, n_q
+    elif kind in ("bottom_right", "band"):
+        causal, n_k = "bottom_right", max(n_k, n_q)
+        if kind == "band":
+            window = rnd.randint(40, 900)
+    pad = rnd.choice([0, 8, 64])   # row stride d + pad
+    x = make_case(batch, n_q, n_k, d, torch.bfloat16, seed=200 + seed, grad_std=0.1)
+    if pad:
+        for name in list(x):
+            t = x[name]
+            wide = torch.zeros(t.shape[0], t.shape[1], d + pad, dtype=t.dtype, device=t.device)
+            wide[..., :d] = t
+            x[name] = wide[..., :d]
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal, window)
+    if pad:
+        wide = torch.zeros(batch, n_q, d + pad, dtype=x["O"].dtype, device="cuda")
+        wide[..., :d] = x["O"]
+        x["O"] = wide[..., :d]
+    fast = run_fhog(x, scale, causal, window=window, impl="bf16", return_stats=True)
+    slow = run_fhog(x, scale, causal, window=window, impl="fp32", return_stats=True)
+    e = errors(fast[:4], slow[:4])
+    assert max(e.values()) < 1.5e-2, (e, d, batch, n_q, n_k, kind, window, pad)
+    for a, b, name in zip(fast[4], slow[4], ("d", "dd", "b")):
+        assert normalised_max_error(a, b) < 1e-2, name
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("impl", ["bf16", "fp32"])
 @pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
