@@ -8,8 +8,8 @@
 //   consumers (4 waves, same rows): the second-level products of the PREVIOUS block on MFMA
 //     (4 contractions in pass 3, 3 in pass 4) into the fp32 output accumulators, plus all
 //     global -> LDS staging of the streamed tiles.
-// The consumer runs one block behind the producer, so the VALU phase of the producer and the MFMA
-// phase of the consumer on the same SIMD overlap in hardware; each wave fits 256 registers.
+// The consumer runs one block behind the producer, so the VALU-heavy end of the producer's block and the MFMAs of
+// the consumer on the same SIMD can overlap; each wave fits 256 registers.
 // One barrier per 32-row step. LDS: 3-stage ring of streamed tiles + double-buffered operand tiles.
 #include "fhog_bf16_util.h"
 
@@ -38,7 +38,8 @@ struct PCSmem {
 // The five first-level products are issued as a stream of 32 k-steps (8 each for K, V, ddK, ddV);
 // the elementwise work of the block is cut into 2-element pieces that are placed right behind the
 // MFMAs in the SAME wave's instruction stream, where they execute in the shadow of the matrix pipe
-// (VALU work of another wave does not overlap an MFMA on this hardware; work of the same wave does):
+// (VALU work of another wave overlaps an MFMA only in part: both go through the SIMD's one vector issue port, and a
+// pure-MFMA wave next to a pure-VALU wave of the same length takes 1.35x the time of either):
 //   steps  0.. 7  A = K  : S += K Q^T, ddS += K ddQ^T
 //   steps  8..15  A = V  : dP += V dO^T          + P = exp2(S c - L)
 //   steps 16..23  A = ddK: ddS += ddK Q^T        + u = dP - d, dS = P u, v = dP dd + b
