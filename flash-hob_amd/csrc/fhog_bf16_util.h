@@ -293,12 +293,21 @@ __host__ __forceinline__ unsigned grid_blocks(int n_tiles, int batch) {
   return (unsigned)(rounds * 8 * tiles_per_xcd);
 }
 // Returns false when the id falls beyond the last slice or tile.
-__device__ __forceinline__ bool decode_block(int n_tiles, int batch, bool heavy_first, int& bh, int& tile) {
+// tile_major: the slices that share an XCD advance through their tiles together (ids enumerate tile 0 of every
+// slice, then tile 1 of every slice, ...) instead of one slice after the other. With a mask the work of a tile grows
+// with its index; heaviest-first over ALL workgroups of the XCD is what lets the light tiles at the end fill the
+// gaps (one slice after the other leaves the last slice's heavy tiles alone at the end whenever the XCD holds more
+// resident workgroups than a slice has tiles). All workgroups stream the other side from its first tile on, so the
+// slices still move through L2 together.
+__device__ __forceinline__ bool decode_block(int n_tiles, int batch, bool heavy_first, bool tile_major, int& bh, int& tile) {
   const int id = blockIdx.x;
   const int xcd = id & 7, slot = id >> 3;
   const int xs = xcds_per_slice(batch), per_round = 8 / xs, tiles_per_xcd = (n_tiles + xs - 1) / xs;
-  bh = xcd / xs + per_round * (slot / tiles_per_xcd);
-  tile = (slot % tiles_per_xcd) * xs + xcd % xs;
+  const int rounds = (batch + per_round - 1) / per_round;   // slices this XCD (group) serves
+  const int r = tile_major ? slot % rounds : slot / tiles_per_xcd;
+  const int t = tile_major ? slot / rounds : slot % tiles_per_xcd;
+  bh = xcd / xs + per_round * r;
+  tile = t * xs + xcd % xs;
   if (bh >= batch || tile >= n_tiles) return false;
   if (heavy_first) tile = n_tiles - 1 - tile;
   return true;

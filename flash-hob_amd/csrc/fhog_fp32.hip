@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   // then does the same amount of work, whatever their number.
   const int n_tiles = (n_sta + TR * nw - 1) / (TR * nw);
   int bh, unit;
-  if (!bf16k::decode_block(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch, false, bh, unit)) return;
+  if (!bf16k::decode_block(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch, false, false, bh, unit)) return;
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const int64_t sta_ld = KSIDE ? p.stride_kn : p.stride_qn, str_ld = KSIDE ? p.stride_qn : p.stride_kn;
   // stationary tensors: Q, ddQ, dO | K, ddK, V, ddV; streamed tensors: K, ddK, V, ddV | Q, ddQ, dO
