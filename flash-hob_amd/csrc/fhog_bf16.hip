@@ -167,6 +167,9 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
       //   ddV: E += ddV dO^T           + acc += P (ddS u - t)                      (pass 2)
       //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
       //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
+      // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
+      // ddK; ddP = P (ddS scale - dd), z = P (ddS u scale - v) behind ddV; dS' = P E + z in the tail), packs the four
+      // tiles to 16 bits and goes on to the second-level products.
       constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
       constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
       f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
