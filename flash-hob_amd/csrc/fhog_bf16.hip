@@ -20,6 +20,7 @@
 // accumulators, rounded to 16 bits, are the B operands of those products as they stand (contraction over the
 // streamed rows), the A operands are transposing reads of the staged tiles in the same row order. At d = 128
 // the output accumulators alone take 128 registers and the work is split over producer and consumer waves.
+
 #include "fhog_bf16_util.h"
 
 namespace fhog {
@@ -63,9 +64,10 @@ __global__ void __launch_bounds__(256) combine_out(const float* part, int n_spli
   *reinterpret_cast<u32x2_t*>(out1 + o) = pack4<F16>(b[0], b[1], b[2], b[3]);
 }
 
-template <bool F16, int D, int PASS, int MASK>
-__global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
+template <bool F16, int D, int PASS, int MASK, int NW = 4>
+__global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int ROWS = 32 * NW;
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
   constexpr int TILE = TS * 2 * D;
   constexpr int STAGE = NT * TILE;
@@ -73,12 +75,12 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
 
   // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
   int bh, tile, split = 0;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch * p.n_split, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
   if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
-  const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int q0 = tile * ROWS, qw = q0 + 32 * wave, qi = qw + n;
   const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
@@ -136,13 +138,23 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
 
   const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
   int j_begin, j_end;  // key tiles this workgroup visits
-  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
+  geo.tile_range(q0, ROWS, j_begin, j_end);
   if (p.n_split > 1) split_range(split, p.n_split, j_begin, j_end);
+  // staging: four waves share the rows of a tile; with eight waves each group of four takes half of the tensors
+  constexpr int NLD = NW == 8 ? NT / 2 : NT;
+  const int half = NW == 8 ? wave >> 2 : 0;
+  const __bf16* srcl[NLD];
+#pragma unroll
+  for (int x = 0; x < NLD; x++) {   // wave-uniform, and the staging instruction wants it in scalar registers
+    const uint64_t a = (uint64_t)(NW == 8 ? (half ? src[NT / 2 + x < NT ? NT / 2 + x : 0] : src[x]) : src[x]);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    srcl[x] = (const __bf16*)(((uint64_t)hi << 32) | lo);
+  }
   Dma<D> dma;
-  dma.init(p.stride_kn, wave, lane);
-  const uint32_t ring_lds = lds_addr(smem);
+  dma.init(p.stride_kn, wave & 3, lane);
+  const uint32_t ring_lds = lds_addr(smem) + half * NLD * TILE;
   if (j_begin < j_end)
-    dma.template issue_all<NT>(ring_lds + (j_begin & 1) * STAGE, TILE, src, (int64_t)j_begin * TS * p.stride_kn, wave, p.n_k - j_begin * TS);
+    dma.template issue_all<NLD>(ring_lds + (j_begin & 1) * STAGE, TILE, srcl, (int64_t)j_begin * TS * p.stride_kn, wave & 3, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
@@ -150,7 +162,7 @@ __global__ void __launch_bounds__(256, 2) q_sweep_bf16(Params p) {
     if (j + 1 < j_end) {
       const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
       const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-      dma.template issue_all<NT>(dst, TILE, src, adv, wave, p.n_k - (j + 1) * TS);
+      dma.template issue_all<NLD>(dst, TILE, srcl, adv, wave & 3, p.n_k - (j + 1) * TS);
     }
     const int k0 = j * TS;
     const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
@@ -566,6 +578,20 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   const bool split = p.n_split > 1;
   const int64_t rows_q = (int64_t)p.batch * p.n_q, rows_k = (int64_t)p.batch * p.n_k;
   hipError_t e;
+  // Passes 2 and 5 with plenty of workgroups run 256 rows per workgroup (8 waves, one workgroup per CU): each staged
+  // tile then serves twice the rows, i.e. half the staging loads per row (cfg2: pass 2 -7 %). Pass 1 (two tensors,
+  // three workgroups per CU), d = 64 (measured slower or equal) and small launches keep 128 rows.
+  const unsigned g8 = grid_blocks((p.n_q + 255) / 256, slices);
+  if (D == 128 && !split && g8 >= 512 && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
+    const auto launch8 = [&](auto kernel, int smem) {
+      const hipError_t e8 = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e8 != hipSuccess) return e8;
+      hipLaunchKernelGGL(kernel, dim3(g8), dim3(512), smem, s, p);
+      return hipGetLastError();
+    };
+    if (pass == FHOG_PASS_B) return launch8(q_sweep_bf16<F16, D, 2, MASK, 8>, 2 * 4 * tile);
+    return launch8(q_sweep_bf16<F16, D, 5, MASK, 8>, 2 * 4 * tile);
+  }
   switch (pass) {
     case FHOG_PASS_DD:
       e = launch_sweep(q_sweep_bf16<F16, D, 1, MASK>, gq, 2 * 2 * tile, s, p);

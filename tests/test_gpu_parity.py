@@ -321,6 +321,26 @@ def test_split_launches_on_random_shapes_against_the_fp32_family(seed):
         assert normalised_max_error(a, b) < 1e-2, name
 
 
+@pytest.mark.parametrize("fused_stats", [False, True])
+@pytest.mark.parametrize("case", [(130, 1000, 1000, "causal", None, torch.bfloat16), (128, 1025, 700, "none", None, torch.float16),
+                                  (171, 770, 1100, "bottom_right", 300, torch.bfloat16), (64, 2050, 520, "none", None, torch.bfloat16)])
+def test_many_slices_d128_statistics_in_256_row_workgroups(case, fused_stats):
+    """At d = 128, launches of the b and dd+b sweeps with at least 512 workgroups of 256 query rows use those (8 waves)
+    instead of 128-row workgroups: ragged lengths (last workgroup partly or, for its upper waves, wholly past the end),
+    masks and dtypes against the fp32-MFMA kernels, statistics included."""
+    batch, n_q, n_k, kind, window, dtype = case
+    causal = {"none": False, "causal": True, "bottom_right": "bottom_right"}[kind]
+    x = make_case(batch, n_q, n_k, 128, dtype, seed=77, grad_std=0.1)
+    scale = 128 ** -0.5
+    x = with_caches(x, scale, causal, window)
+    fast = run_fhog(x, scale, causal, window=window, impl="bf16", fused_stats=fused_stats, return_stats=True)
+    slow = run_fhog(x, scale, causal, window=window, impl="fp32", return_stats=True)
+    e = errors(fast[:4], slow[:4])
+    assert max(e.values()) < 1.5e-2, e
+    for a, b, name in zip(fast[4], slow[4], ("d", "dd", "b")):
+        assert normalised_max_error(a, b) < 1e-2, name
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("impl", ["bf16", "fp32"])
 @pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
