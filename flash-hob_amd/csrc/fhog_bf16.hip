@@ -112,6 +112,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   }
   const float dd = (PASS == 2 || PASS == 3) ? p.ws_dd[row] : 0.f;
   const float b = PASS == 3 ? p.ws_b[row] : 0.f;
+  const float kc = __builtin_fmaf(dd, dsum, b);   // per-row constant of dP' = E + (ddS - dd)(dP - d) - kc (passes 2, 3)
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
   // PASS 3 (d = 64): the second-level products follow in the same wave, with the S-shaped tiles as B operands
   // straight from the registers; lane = query, registers = output columns
@@ -175,12 +176,12 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
       //   K  : S += K Q^T, ddS += K ddQ^T
       //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
-      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale, t = dP dd   (pass 2; fused: u only)
-      //   ddV: E += ddV dO^T           + acc += P (ddS u - t)                      (pass 2)
+      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = dP - d   (pass 2; fused: u scale)
+      //   ddV: E += ddV dO^T           + acc += P ((ddS - dd) u - dd d)   [= P (ddS u - dP dd)]   (pass 2)
       //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
       //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
       // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
-      // ddK; ddP = P (ddS scale - dd), z = P (ddS u scale - v) behind ddV; dS' = P E + z in the tail), packs the four
+      // ddK; w = ddS scale - dd, ddP = P w, z = P (w u - dd d - b) behind ddV; dS' = P E + z in the tail), packs the four
       // tiles to 16 bits and goes on to the second-level products.
       constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
       constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
@@ -214,13 +215,12 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
             if (PASS == 1) {
               pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
             } else if (PASS == 3) {
-              const float u = dp[r] - dsum;
-              tt[r] = __builtin_fmaf(dp[r], dd, b);   // v = dP dd + b
-              dp[r] = u;
-              us[r] = pv[r] * u;                       // dS (scale applied to the accumulator at the end)
+              dp[r] -= dsum;                           // u
+              us[r] = pv[r] * dp[r];                   // dS (scale applied to the accumulator at the end)
+            } else if (PASS == 2) {
+              us[r] = dp[r] - dsum;                    // u
             } else {
               us[r] = (dp[r] - dsum) * p.scale;
-              if (PASS == 2) tt[r] = dp[r] * dd;
             }
           }
         } else {
@@ -233,10 +233,11 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 2) {
-              red = __builtin_fmaf(pv[r], __builtin_fmaf(dds[r], us[r], -tt[r]), red);
+              red = __builtin_fmaf(pv[r], __builtin_fmaf(__builtin_fmaf(dds[r], p.scale, -dd), us[r], -kc), red);
             } else if (PASS == 3) {
-              const float ddp = pv[r] * __builtin_fmaf(dds[r], p.scale, -dd);
-              tt[r] = pv[r] * __builtin_fmaf(dds[r] * dp[r], p.scale, -tt[r]);   // z = P (ddS u - v)
+              const float w = __builtin_fmaf(dds[r], p.scale, -dd);
+              const float ddp = pv[r] * w;
+              tt[r] = pv[r] * __builtin_fmaf(w, dp[r], -kc);   // z = P (w u - kc)
               if (r & 1) {
                 pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
                 pk_ds[r / 2] = pack2<F16>(us[r - 1], us[r]);
@@ -493,12 +494,10 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
         for (int i = 0; i < 4; i++) {
           const int r = 4 * g + i;
           const float pr = pv[r];
-          const float ddsv = dds[r] * p.scale;
-          const float t1 = ddsv - dd4[i];
-          const float dp2 = __builtin_fmaf(-ddsv, d4[i], __builtin_fmaf(dp[r], t1, e[r]));
-          dds[r] = pr * t1;
-          s[r] = pr * (dp[r] - d4[i]);
-          e[r] = pr * (dp2 - b4[i]);
+          const float w = __builtin_fmaf(dds[r], p.scale, -dd4[i]), u = dp[r] - d4[i];
+          dds[r] = pr * w;
+          s[r] = pr * u;
+          e[r] = pr * (__builtin_fmaf(w, u, e[r]) - __builtin_fmaf(dd4[i], d4[i], b4[i]));   // dP' = E + w u - (dd d + b)
         }
       }
       const bf16x8_t op_ds[2] = {pack_operand<F16>(s, 0), pack_operand<F16>(s, 1)};

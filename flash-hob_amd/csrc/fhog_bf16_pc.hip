@@ -42,8 +42,8 @@ struct PCSmem {
 // pure-MFMA wave next to a pure-VALU wave of the same length takes 1.35x the time of either):
 //   steps  0.. 7  A = K  : S += K Q^T, ddS += K ddQ^T
 //   steps  8..15  A = V  : dP += V dO^T          + P = exp2(S c - L)
-//   steps 16..23  A = ddK: ddS += ddK Q^T        + u = dP - d, dS = P u, v = dP dd + b
-//   steps 24..31  A = ddV: E += ddV dO^T         + ddP = P (ddS - dd), z = P (ddS u - v)
+//   steps 16..23  A = ddK: ddS += ddK Q^T        + u = dP - d, dS = P u
+//   steps 24..31  A = ddV: E += ddV dO^T         + w = ddS - dd, ddP = P w, z = P (w u - k) with k = dd d + b per row
 //   tail                                          dS' = P E + z     [= P (E + dP (ddS - dd) - ddS d - b)]
 // LDS operands are fetched PF steps ahead. Results go to the operand tiles dS, dS', ddP, P.
 
@@ -73,7 +73,8 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
     return KSIDE ? mfma<F16>(resident, staged, acc) : mfma<F16>(staged, resident, acc);
   };
   f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
-  f32x16_t pv, vv, us;
+  f32x16_t pv, us;
+  const float kc = __builtin_fmaf(dd, dsum, b);   // dS' = P (E + w u - kc) with u = dP - d, w = ddS - dd
   uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];
   bf16x8_t a[NB];
 #pragma unroll
@@ -101,12 +102,9 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       }
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
-        const float u0 = dp[r] - dsum, u1 = dp[r + 1] - dsum;
-        pk_ds[r / 2] = pack2<F16>(pv[r] * u0, pv[r + 1] * u1);
-        vv[r] = __builtin_fmaf(dp[r], dd, b);
-        vv[r + 1] = __builtin_fmaf(dp[r + 1], dd, b);
-        us[r] = u0 * scale;
-        us[r + 1] = u1 * scale;
+        us[r] = dp[r] - dsum;
+        us[r + 1] = dp[r + 1] - dsum;
+        pk_ds[r / 2] = pack2<F16>(pv[r] * us[r], pv[r + 1] * us[r + 1]);
       }
       // the eight registers of a k-step are complete every 8 / EPK steps: hand them off right away, so that the
       // writes travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
@@ -115,10 +113,11 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       e = mm(a[c], re[kk], e);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
-        pk_ddp[r / 2] = pack2<F16>(pv[r] * __builtin_fmaf(dds[r], scale, -dd), pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd));
+        const float w0 = __builtin_fmaf(dds[r], scale, -dd), w1 = __builtin_fmaf(dds[r + 1], scale, -dd);
+        pk_ddp[r / 2] = pack2<F16>(pv[r] * w0, pv[r + 1] * w1);
         pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
-        vv[r] = pv[r] * __builtin_fmaf(dds[r], us[r], -vv[r]);              // z
-        vv[r + 1] = pv[r + 1] * __builtin_fmaf(dds[r + 1], us[r + 1], -vv[r + 1]);
+        us[r] = pv[r] * __builtin_fmaf(w0, us[r], -kc);              // z
+        us[r + 1] = pv[r + 1] * __builtin_fmaf(w1, us[r + 1], -kc);
       }
       if ((EPK * (kk + 1)) % 8 == 0) {
         sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, (EPK * kk) / 8, lane);
@@ -129,7 +128,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
   }
 #pragma unroll
   for (int r = 0; r < 16; r += 2)
-    pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], vv[r]), __builtin_fmaf(pv[r + 1], e[r + 1], vv[r + 1]));
+    pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], us[r]), __builtin_fmaf(pv[r + 1], e[r + 1], us[r + 1]));
   sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 0, lane);
   sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 1, lane);
 }
