@@ -176,8 +176,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
       //   K  : S += K Q^T, ddS += K ddQ^T
       //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
-      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = dP - d   (pass 2; fused: u scale)
-      //   ddV: E += ddV dO^T           + acc += P ((ddS - dd) u - dd d)   [= P (ddS u - dP dd)]   (pass 2)
+      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale (fused)
+      //   ddV: E += ddV dO^T           + acc += P (ddS - dd) u   (pass 2: with u = dP - d and E' = E - dd d from accumulators
+      //                                  that start at the row constants, acc ends as sum P (E' + (ddS - dd) u) = sum P (E + ddS u - dP dd))
       //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
       //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
       // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
@@ -186,6 +187,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
       constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
       f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
+      if (PASS == 2) {   // u = dP - d and E' = E - kc straight from the matrix pipe (in pass 3 this measured slower)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dp[r] = -dsum, e[r] = -kc;
+      }
       uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];   // PASS 3: packed dS, dS', ddP, P (registers 2i, 2i+1)
       bf16x8_t a[NB];
 #pragma unroll
@@ -216,10 +221,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
               pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
             } else if (PASS == 3) {
               dp[r] -= dsum;                           // u
-              us[r] = pv[r] * dp[r];                   // dS (scale applied to the accumulator at the end)
-            } else if (PASS == 2) {
-              us[r] = dp[r] - dsum;                    // u
-            } else {
+              us[r] = pv[r] * dp[r];                   // dS = P u (scale applied to the accumulator at the end)
+            } else if (PASS == 5) {
               us[r] = (dp[r] - dsum) * p.scale;
             }
           }
@@ -233,7 +236,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
 #pragma unroll
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 2) {
-              red = __builtin_fmaf(pv[r], __builtin_fmaf(__builtin_fmaf(dds[r], p.scale, -dd), us[r], -kc), red);
+              red = __builtin_fmaf(pv[r] * __builtin_fmaf(dds[r], p.scale, -dd), dp[r], red);   // P w u
             } else if (PASS == 3) {
               const float w = __builtin_fmaf(dds[r], p.scale, -dd);
               const float ddp = pv[r] * w;
@@ -370,7 +373,7 @@ template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
-  constexpr int STAT = 4 * TS * 4;         // L log2(e), d, dd, b of the 32 staged queries
+  constexpr int STAT = 4 * TS * 4;         // L log2(e), -d, dd, -(dd d + b) of the 32 staged queries
   constexpr int STAGE = 3 * TILE + STAT;   // Q, ddQ, dO tiles, statistics
 
   int bh, tile, split = 0;
@@ -417,14 +420,26 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   Dma<D> dma;
   dma.init(p.stride_qn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-  float stat_reg = 0.f;
+  float stat_reg = 0.f, stat_d = 0.f, stat_dd = 0.f;
   // The statistic is loaded (a global, not generic, load) before the staging loads of a step and first touched at
-  // the end of the step, so the wave never waits for it in between.
+  // the end of the step, so the wave never waits for it in between. Staged per query: L log2(e), -d, dd and
+  // -(dd d + b), the values the accumulators of dP and E start from (the threads of the last group load d and dd too).
   auto load_stat = [&](int q_base) {
-    if (tid < 4 * TS) stat_reg = *(global_f32_ptr)(stat_src + min(q_base + (tid & (TS - 1)), p.n_q - 1));
+    if (tid < 4 * TS) {
+      const int q = min(q_base + (tid & (TS - 1)), p.n_q - 1);
+      stat_reg = *(global_f32_ptr)(stat_src + q);
+      if (tid >= 3 * TS) {
+        stat_d = *(global_f32_ptr)(p.ws_d + (int64_t)bh * p.n_q + q);
+        stat_dd = *(global_f32_ptr)(p.ws_dd + (int64_t)bh * p.n_q + q);
+      }
+    }
   };
   auto store_stat = [&](char* stage_base) {
-    if (tid < 4 * TS) reinterpret_cast<float*>(stage_base + 3 * TILE)[tid] = (tid < TS) ? stat_reg * kLog2e : stat_reg;
+    if (tid < 4 * TS) {
+      const int g = tid / TS;
+      reinterpret_cast<float*>(stage_base + 3 * TILE)[tid] =
+          g == 0 ? stat_reg * kLog2e : g == 1 ? -stat_reg : g == 2 ? stat_reg : -__builtin_fmaf(stat_dd, stat_d, stat_reg);
+    }
   };
   if (t_begin < t_end) {
     load_stat(t_begin * TS);
@@ -450,7 +465,16 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
       const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
       // five first-level products in one stream of KK k-steps; the three staged operands of step kk + 1 are
       // fetched before the MFMAs of step kk: S = Q K^T, ddS = ddQ K^T + Q ddK^T, dP = dO V^T, E = dO ddV^T
-      f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
+      // register 4g + i belongs to query qb + 8g + 4h + i: its statistics come from the staged arrays. The accumulators
+      // of dP and E start at -d and -(dd d + b): u = dP - d and E' = E - dd d - b come straight from the matrix pipe.
+      f32x16_t s = {0}, dds = {0}, dp, e;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x4_t md4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
+        const f32x4_t mk4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
+#pragma unroll
+        for (int i = 0; i < 4; i++) dp[4 * g + i] = md4[i], e[4 * g + i] = mk4[i];
+      }
       bf16x8_t a[2][3];
 #pragma unroll
       for (int x = 0; x < 3; x++) a[0][x] = lds_read128(stage + x * TILE, aoff[0]);
@@ -469,7 +493,6 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
         e = mfma<F16>(a[c][2], ddVb[kk], e);
         __builtin_amdgcn_sched_barrier(0);
       }
-      // register 4g + i belongs to query qb + 8g + 4h + i: its statistics come from the staged arrays
       f32x16_t pv;
 #pragma unroll
       for (int g = 0; g < 4; g++) {
@@ -487,17 +510,14 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
       // dS -> s, dS' -> e, ddP -> dds (in place; scale on dS, dS' is applied to the accumulators at the end)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
         const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
-        const f32x4_t b4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int r = 4 * g + i;
           const float pr = pv[r];
-          const float w = __builtin_fmaf(dds[r], p.scale, -dd4[i]), u = dp[r] - d4[i];
-          dds[r] = pr * w;
-          s[r] = pr * u;
-          e[r] = pr * (__builtin_fmaf(w, u, e[r]) - __builtin_fmaf(dd4[i], d4[i], b4[i]));   // dP' = E + w u - (dd d + b)
+          dds[r] = pr * __builtin_fmaf(dds[r], p.scale, -dd4[i]);   // ddP = P (ddS - dd)
+          s[r] = pr * dp[r];                                         // dS = P u
+          e[r] = __builtin_fmaf(pr, e[r], dds[r] * dp[r]);           // dS' = P (E' + (ddS - dd) u)
         }
       }
       const bf16x8_t op_ds[2] = {pack_operand<F16>(s, 0), pack_operand<F16>(s, 1)};

@@ -42,9 +42,11 @@ struct PCSmem {
 // pure-MFMA wave next to a pure-VALU wave of the same length takes 1.35x the time of either):
 //   steps  0.. 7  A = K  : S += K Q^T, ddS += K ddQ^T
 //   steps  8..15  A = V  : dP += V dO^T          + P = exp2(S c - L)
-//   steps 16..23  A = ddK: ddS += ddK Q^T        + u = dP - d, dS = P u
-//   steps 24..31  A = ddV: E += ddV dO^T         + w = ddS - dd, ddP = P w, z = P (w u - k) with k = dd d + b per row
-//   tail                                          dS' = P E + z     [= P (E + dP (ddS - dd) - ddS d - b)]
+//   steps 16..23  A = ddK: ddS += ddK Q^T        + dS = P u
+//   steps 24..31  A = ddV: E' += ddV dO^T        + w = ddS - dd, ddP = P w, z = ddP u
+//   tail                                          dS' = P E' + z     [= P (E + dP (ddS - dd) - ddS d - b)]
+// with u = dP - d and E' = E - (dd d + b) straight from the matrix pipe: the accumulators of dP and E start at the
+// (per-lane) row constants -d and -(dd d + b) instead of zero.
 // LDS operands are fetched PF steps ahead. Results go to the operand tiles dS, dS', ddP, P.
 
 // registers 8t .. 8t+7 of one S-shaped tile, given as packed pairs pk[4t] .. pk[4t+3]: one ds_write_b128, so that the
@@ -72,9 +74,10 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
   const auto mm = [](bf16x8_t staged, bf16x8_t resident, f32x16_t acc) {
     return KSIDE ? mfma<F16>(resident, staged, acc) : mfma<F16>(staged, resident, acc);
   };
-  f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0};
-  f32x16_t pv, us;
+  f32x16_t s = {0}, dds = {0}, dp, e, pv, z;   // dp holds u, e holds E'
   const float kc = __builtin_fmaf(dd, dsum, b);   // dS' = P (E + w u - kc) with u = dP - d, w = ddS - dd
+#pragma unroll
+  for (int r = 0; r < 16; r++) dp[r] = -dsum, e[r] = -kc;
   uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];
   bf16x8_t a[NB];
 #pragma unroll
@@ -101,11 +104,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
         for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
       }
 #pragma unroll
-      for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
-        us[r] = dp[r] - dsum;
-        us[r + 1] = dp[r + 1] - dsum;
-        pk_ds[r / 2] = pack2<F16>(pv[r] * us[r], pv[r + 1] * us[r + 1]);
-      }
+      for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) pk_ds[r / 2] = pack2<F16>(pv[r] * dp[r], pv[r + 1] * dp[r + 1]);
       // the eight registers of a k-step are complete every 8 / EPK steps: hand them off right away, so that the
       // writes travel while the matrix pipe is busy instead of queueing up behind the consumers' reads at the end
       if ((EPK * (kk + 1)) % 8 == 0) sop_write_pk(sop + 0 * SOP_TILE, pk_ds, (EPK * kk) / 8, lane);
@@ -113,11 +112,11 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
       e = mm(a[c], re[kk], e);
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
-        const float w0 = __builtin_fmaf(dds[r], scale, -dd), w1 = __builtin_fmaf(dds[r + 1], scale, -dd);
-        pk_ddp[r / 2] = pack2<F16>(pv[r] * w0, pv[r + 1] * w1);
+        const float ddp0 = pv[r] * __builtin_fmaf(dds[r], scale, -dd), ddp1 = pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd);
+        pk_ddp[r / 2] = pack2<F16>(ddp0, ddp1);
         pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
-        us[r] = pv[r] * __builtin_fmaf(w0, us[r], -kc);              // z
-        us[r + 1] = pv[r + 1] * __builtin_fmaf(w1, us[r + 1], -kc);
+        z[r] = ddp0 * dp[r];
+        z[r + 1] = ddp1 * dp[r + 1];
       }
       if ((EPK * (kk + 1)) % 8 == 0) {
         sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, (EPK * kk) / 8, lane);
@@ -128,7 +127,7 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
   }
 #pragma unroll
   for (int r = 0; r < 16; r += 2)
-    pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], us[r]), __builtin_fmaf(pv[r + 1], e[r + 1], us[r + 1]));
+    pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], z[r]), __builtin_fmaf(pv[r + 1], e[r + 1], z[r + 1]));
   sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 0, lane);
   sop_write_pk(sop + 1 * SOP_TILE, pk_ds2, 1, lane);
 }
