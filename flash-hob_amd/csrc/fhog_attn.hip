@@ -234,14 +234,16 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
     if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
     if (!geo.dead(k0, qw)) {
       const char* stage = smem + (j & 1) * STAGE;
-      f32x16_t s[1] = {f32x16_t{0}}, dp[1] = {f32x16_t{0}};
+      f32x16_t s[1] = {f32x16_t{0}}, dp[1];
+#pragma unroll
+      for (int r = 0; r < 16; r++) dp[0][r] = -dsum;        // the accumulator ends as dP - d
       const bf16x8_t* const rq[1] = {Qb};
       const bf16x8_t* const rdo[1] = {dOb};
       first_level<F16, D, 1>(stage, aoff, rq, s);           // S^T  = K Q^T
-      first_level<F16, D, 1>(stage + TILE, aoff, rdo, dp);  // dP^T = V dO^T
+      first_level<F16, D, 1>(stage + TILE, aoff, rdo, dp);  // dP^T = V dO^T - d
       f32x16_t ds;
 #pragma unroll
-      for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * (dp[0][r] - dsum);
+      for (int r = 0; r < 16; r++) ds[r] = __builtin_amdgcn_exp2f(s[0][r] * c_scale_log2 - l_log2) * dp[0][r];
       if (masked) {
         keep_branch();
 #pragma unroll

@@ -533,7 +533,9 @@ __device__ __forceinline__ void produce_first(const char* stage, char* sop, cons
   int aoff[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
-  f32x16_t s = {0}, dp = {0}, pv;
+  f32x16_t s = {0}, dp, pv;   // the accumulator of dP starts at -d: dp ends as dP - d
+#pragma unroll
+  for (int r = 0; r < 16; r++) dp[r] = -dsum;
   bf16x8_t a[NB];
 #pragma unroll
   for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + (i / KK) * TILE, aoff[i % KK]);
@@ -559,7 +561,7 @@ __device__ __forceinline__ void produce_first(const char* stage, char* sop, cons
   uint32_t pk_ds[8], pk_p[8];
 #pragma unroll
   for (int r = 0; r < 16; r += 2) {
-    pk_ds[r / 2] = pack2<F16>(pv[r] * (dp[r] - dsum), pv[r + 1] * (dp[r + 1] - dsum));
+    pk_ds[r / 2] = pack2<F16>(pv[r] * dp[r], pv[r + 1] * dp[r + 1]);
     pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
   }
 #pragma unroll
