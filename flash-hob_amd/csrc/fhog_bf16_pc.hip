@@ -328,7 +328,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 __device__ __forceinline__ int sop_tr_lane_off(int s, int lane) {
   const int i = lane & 15, b = (lane >> 4) & 1, h = lane >> 5, cg = i & 3;
   const int r = 8 * s + 4 * h + (i >> 2);
-  return r * 64 + (((2 * b + (cg & 1)) ^ ((r >> 2) & 3)) << 4) + 8 * (cg >> 1);
+  return r * 64 + (((2 * b + (cg & 1)) ^ sop_swz(r)) << 4) + 8 * (cg >> 1);
 }
 
 template <bool F16, int D, int MASK>
