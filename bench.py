@@ -228,8 +228,8 @@ def main():
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), keyed by (workload, pass). None until measured for that kernel.
-TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((475.5 + 64.0) * 2 ** 20),
-                 ("cfg2_bf16_causal_4096_d128", 4): int((373.7 + 64.0) * 2 ** 20)}
+TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((510.1 + 64.4) * 2 ** 20),
+                 ("cfg2_bf16_causal_4096_d128", 4): int((372.1 + 64.0) * 2 ** 20)}
 
 if __name__ == "__main__":
     main()
