@@ -12,8 +12,8 @@
 //
 // The kernels of this file are single-role: a workgroup is 256 threads = 4 wave64 owning 128 stationary rows,
 // two workgroups per CU (the b sweeps at d = 128 also exist with 8 waves and 256 rows, one workgroup per CU, for
-// launches with enough workgroups: half the staging loads per row). Each wave keeps its 32 rows in registers as MFMA B operands (Q, ddQ and, from pass 2
-// on, dO; K, ddK, V, ddV in pass 4); the other side streams through a two-stage LDS ring of 32-row tiles filled by
+// launches with enough workgroups: half the staging loads per row). Each wave keeps its 32 rows in registers as
+// MFMA B operands (Q, ddQ and, from pass 2 on, dO; K, ddK, V, ddV in pass 4); the other side streams through a two-stage LDS ring of 32-row tiles filled by
 // direct global->LDS loads. First-level products are computed with the streamed rows as M and the stationary
 // rows as N, so every lane owns ONE stationary row: in the Q-tiled sweeps L, d, dd, b are per-lane scalars and a
 // row sum is a per-lane partial sum, reduced once at the end with a single cross-half shuffle.
@@ -178,8 +178,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       //   K  : S += K Q^T, ddS += K ddQ^T
       //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
       //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale (fused)
-      //   ddV: E += ddV dO^T           + acc += P (ddS - dd) u   (pass 2: with u = dP - d and E' = E - dd d from accumulators
-      //                                  that start at the row constants, acc ends as sum P (E' + (ddS - dd) u) = sum P (E + ddS u - dP dd))
+      //   ddV: E += ddV dO^T           + acc += P (ddS - dd) u   (pass 2: u = dP - d and E' = E - dd d come from
+      //                                  accumulators that start at the row constants; with the tail, acc ends as
+      //                                  sum P (E' + (ddS - dd) u) = sum P (E + ddS u - dP dd))
       //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
       //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
       // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
