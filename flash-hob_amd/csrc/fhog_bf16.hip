@@ -584,10 +584,10 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
 }
 
 template <typename K>
-hipError_t launch_sweep(K kernel, unsigned grid, int smem, hipStream_t s, const Params& p) {
+hipError_t launch_sweep(K kernel, unsigned grid, int smem, hipStream_t s, const Params& p, unsigned threads = 256) {
   const hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, s, p);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
@@ -604,14 +604,8 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   // three workgroups per CU), d = 64 (measured slower or equal) and small launches keep 128 rows.
   const unsigned g8 = grid_blocks((p.n_q + 255) / 256, slices);
   if (D == 128 && !split && g8 >= 512 && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
-    const auto launch8 = [&](auto kernel, int smem) {
-      const hipError_t e8 = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-      if (e8 != hipSuccess) return e8;
-      hipLaunchKernelGGL(kernel, dim3(g8), dim3(512), smem, s, p);
-      return hipGetLastError();
-    };
-    if (pass == FHOG_PASS_B) return launch8(q_sweep_bf16<F16, D, 2, MASK, 8>, 2 * 4 * tile);
-    return launch8(q_sweep_bf16<F16, D, 5, MASK, 8>, 2 * 4 * tile);
+    if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
+    return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
   }
   switch (pass) {
     case FHOG_PASS_DD:
