@@ -120,17 +120,16 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
       f32x16_t s[1] = {f32x16_t{0}};
       const bf16x8_t* const res[1] = {Qb};
       first_level<F16, D, 1>(stage, aoff, res, s);  // S^T: s[r] = (key k0 + 8(r/4) + 4h + r%4, query qi)
-      f32x16_t x;
-#pragma unroll
-      for (int r = 0; r < 16; r++) x[r] = s[0][r] * c_scale_log2;
+      f32x16_t x = s[0];   // raw scores; the scale (positive) goes into the exponent's FMA, maxima commute with it
       if (masked) {
         keep_branch();
 #pragma unroll
         for (int r = 0; r < 16; r++) x[r] = in_limits(r, lo, hi) ? x[r] : -INFINITY;
       }
-      float tmax = x[0];
+      float tmax = fmaxf(fmaxf(x[0], x[1]), x[2]);
 #pragma unroll
-      for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, x[r]);
+      for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, x[r]), x[r + 1]);
+      tmax = fmaxf(tmax, x[15]) * c_scale_log2;
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
       // The running maximum follows the row maximum only in jumps of more than kMaxSlack (in log2 units): P may then
       // reach 2^kMaxSlack instead of 1, which costs no precision in a 16-bit float or in the fp32 sums, and the output
@@ -143,7 +142,7 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
       float rs = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        x[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
+        x[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r], c_scale_log2, -m_ref));
         rs += x[r];
       }
       l = __builtin_fmaf(l, alpha, rs);
