@@ -527,11 +527,13 @@ def test_peak_memory_is_linear_in_n():
     assert sizes[8192] <= 4.2 * sizes[2048]
 
 
-def test_hip_graph_capture_and_replay():
+@pytest.mark.parametrize("batch,n", [(4, 512), (128, 1024)])
+def test_hip_graph_capture_and_replay(batch, n):
     """The library only enqueues kernels on the caller's stream: a captured call replays to the same bits, also after
-    the inputs changed in place and with eager work in between."""
+    the inputs changed in place and with eager work in between. The small case runs split launches with their combine
+    kernels, the large one the 256-row statistics workgroups."""
     from fhog import BwdBwdPlan
-    x = with_caches(make_case(4, 512, 512, 128, torch.bfloat16, seed=17, grad_std=0.1), 128 ** -0.5, True)
+    x = with_caches(make_case(batch, n, n, 128, torch.bfloat16, seed=17, grad_std=0.1), 128 ** -0.5, True)
     plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 128 ** -0.5, causal=True)
     eager = [t.clone() for t in plan.run()]
     torch.cuda.synchronize()
