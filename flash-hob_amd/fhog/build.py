@@ -27,7 +27,7 @@ HIPCC_FLAGS = [
     # packed-fp32 VALU forms are kept out of every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-] + __import__("os").environ.get("FHOG_EXTRA", "").split()
+] + os.environ.get("FHOG_EXTRA", "").split()   # extra hipcc flags for experiments
 
 
 def hipcc() -> str:
