@@ -603,9 +603,11 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   // tile then serves twice the rows, i.e. half the staging loads per row (cfg2: pass 2 -7 %). Pass 1 (two tensors,
   // three workgroups per CU), d = 64 (measured slower or equal) and small launches keep 128 rows.
   const unsigned g8 = grid_blocks((p.n_q + 255) / 256, slices);
-  if (D == 128 && !split && g8 >= 512 && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
-    if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
-    return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
+  if constexpr (D == 128) {
+    if (!split && g8 >= 512 && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
+      if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
+      return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
+    }
   }
   switch (pass) {
     case FHOG_PASS_DD:
