@@ -187,7 +187,8 @@ int validate_attn(const fhog_attn_args* a, int backward) {
   if (const int rc = check_mask(a->causal, a->window, a->n_q, a->n_k)) return rc;
   if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
     return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128}");
-  if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
+  // the forward takes the running maximum of the raw scores and scales it afterwards, which needs scale > 0
+  if (!isfinite(a->scale) || a->scale <= 0.f) return fail(FHOG_E_SCALE, "scale must be finite and positive (got %g)", (double)a->scale);
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
   if (a->stride_qn > kMaxRowStride || a->stride_kn > kMaxRowStride) return fail(FHOG_E_STRIDE, "row stride above 2^24 elements");
   if (a->stride_qn % 8 || a->stride_kn % 8 || a->stride_qb % 8 || a->stride_kb % 8)

@@ -176,10 +176,16 @@ struct Dma {
         for (int u = 0; u < PER_WAVE; u++) issue_one(tile_lds + x * tile_stride + (lw + 4 * u) * 1024, off[u], src[x] + adv);
     }
   }
+  // M0 is on the clobber list: the compiler never allocates it, but it does write it ahead of instructions of its own
+  // that read it and may share one such write between several of them; the list tells it that this statement changes
+  // the register in between (clang warns about any reserved register on a clobber list; the warning is switched off here).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
   __device__ __forceinline__ static void issue_one(uint32_t lds, uint32_t off, const __bf16* src) {
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory");  // M0 is reserved: the compiler keeps nothing in it
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
   }
+#pragma clang diagnostic pop
 };
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // s_waitcnt vmcnt(0) as a builtin (gfx9 encoding: vmcnt 0, expcnt 7, lgkmcnt 15), which the compiler's wait-count

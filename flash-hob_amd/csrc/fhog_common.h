@@ -43,7 +43,8 @@ struct Params {
   int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
   int32_t window;
   // Streamed side split over n_split workgroups per stationary tile (1 = no split): each writes fp32 partial results
-  // to `part` and a combining kernel finishes the pass. Set per pass by the caller of the launchers (d = 64 kernels).
+  // to `part` and a combining kernel finishes the pass. Set per pass by the caller of the launchers (16-bit kernels,
+  // both head dims).
   int32_t n_split;
   float* part;
 };

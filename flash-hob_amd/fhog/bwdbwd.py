@@ -126,8 +126,8 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
             "bottom_right": j <= i + N_K - N_Q, needs N_K >= N_Q. (The reference's Triton path has no causal
             double-backward; its JAX specification has the bottom-right form, ``fhog/jax_refs/jax_impl.py:110-115``.)
         window: sliding-window length in keys on top of a causal mask (same function of the specification):
-            only the ``window`` most recent visible keys stay visible. The 16-bit MFMA kernels take no mask or
-            the plain square causal mask; other masks run on the fp32-MFMA kernels.
+            only the ``window`` most recent visible keys stay visible. Both kernel families take every mask and
+            skip the tiles outside the band.
         impl: None/"auto" | "fp32" | "bf16" - kernel family; "auto" takes the 16-bit MFMA kernels ("bf16": products
             in the tensor type, bf16 or fp16) for 16-bit tensors whose shape they support, the fp32-MFMA kernels
             otherwise.

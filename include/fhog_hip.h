@@ -43,10 +43,10 @@ extern "C" {
 #define FHOG_E_STRIDE (-4)    /* stride smaller than the row / not a multiple of the vector width / row stride > 2^24 */
 #define FHOG_E_ALIGN (-5)     /* pointer not 16-byte aligned */
 #define FHOG_E_CAUSAL (-6)    /* mask not applicable: top-left causal with n_q != n_k, bottom-right with n_k < n_q,
-                                 a window without a causal mask, or a mask the forced kernel family does not take */
+                                 a negative window, or a window without a causal mask */
 #define FHOG_E_PASS (-7)      /* unknown pass id */
 #define FHOG_E_LAUNCH (-8)    /* HIP reported an error at launch */
-#define FHOG_E_SCALE (-9)     /* scale is not finite */
+#define FHOG_E_SCALE (-9)     /* scale is not finite (fhog_attn_fwd / fhog_attn_bwd: not finite or not positive) */
 
 /* pass ids for fhog_bwdbwd_pass */
 #define FHOG_PASS_D 0      /* d_i  = sum_c O_ic dO_ic                         (fhog/triton_bwdbwd.py:580)     */

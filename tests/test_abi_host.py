@@ -89,6 +89,8 @@ def good_attn_args():
     (lambda a: (setattr(a, "stride_qn", (1 << 24) + 8), setattr(a, "stride_qb", 1 << 40)), 0, -4, "2^24"),
     (lambda a: setattr(a, "v", 0x30008), 0, -5, "aligned"),
     (lambda a: setattr(a, "scale", float("inf")), 0, -9, "scale"),
+    (lambda a: setattr(a, "scale", -0.125), 0, -9, "positive"),   # the forward's running maximum needs scale > 0
+    (lambda a: setattr(a, "scale", 0.0), 1, -9, "positive"),
 ])
 def test_attn_validate(L, mutate, backward, code, word):
     a = good_attn_args()
