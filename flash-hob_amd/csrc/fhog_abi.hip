@@ -5,7 +5,14 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "fhog_common.h"
+
+// Workspace of fhog_bwdbwd_static_ws: device memory that belongs to the loaded library, so that the entry point never
+// allocates. Every GPU the library runs on holds its own copy at its own address until the process ends; the name below
+// is only a host-side handle, the address on the current device comes from hipGetSymbolAddress (scratch_on_device).
+static __device__ __align__(256) unsigned char scratch[FHOG_STATIC_WS_BYTES];
 
 namespace {
 
@@ -225,6 +232,26 @@ fhog::AttnParams to_attn_params(const fhog_attn_args* a) {
   return p;
 }
 
+// Address of `scratch` on the current device, looked up once per device (the first call there) and kept.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int scratch_on_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "hipGetDevice: HIP error %d (%s)", (int)e, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(FHOG_E_LAUNCH, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(FHOG_E_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: HIP error %d (%s)", dev, (int)e, hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // concurrent first calls store the same address
+  }
+  *out = ptr;
+  return FHOG_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -313,6 +340,24 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
     if (r != FHOG_OK) return r;
   }
   return FHOG_OK;
+}
+
+int fhog_bwdbwd_static_ws(const fhog_bwdbwd_args* args, void* hip_stream) {
+  if (!args) return fail(FHOG_E_NULL, "args is NULL");
+  void* ws = nullptr;
+  if (const int rc = scratch_on_device(&ws)) return rc;
+  fhog_bwdbwd_args a = *args;   // the caller's ws / ws_bytes are not read
+  a.ws = static_cast<float*>(ws);
+  a.ws_bytes = 0;
+  if (const int rc = validate(&a)) return rc;
+  const size_t need = fhog_bwdbwd_workspace_bytes(a.batch, a.n_q);
+  if (need > (size_t)FHOG_STATIC_WS_BYTES)
+    return fail(FHOG_E_SHAPE,
+                "fhog_bwdbwd_static_ws: batch*n_q = %lld rows need %zu bytes of row statistics, the static workspace holds %zu "
+                "(at most %zu rows); use fhog_bwdbwd with a caller-owned workspace",
+                (long long)(a.batch * a.n_q), need, (size_t)FHOG_STATIC_WS_BYTES, (size_t)FHOG_STATIC_WS_BYTES / 12);
+  a.ws_bytes = FHOG_STATIC_WS_BYTES;   // small launches split their streamed side as far as the rest of the array allows
+  return fhog_bwdbwd(&a, hip_stream);
 }
 
 int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream) {

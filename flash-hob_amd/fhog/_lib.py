@@ -16,7 +16,8 @@ DTYPE_BF16, DTYPE_FP32, DTYPE_FP16 = 0, 1, 2
 IMPL_AUTO, IMPL_FP32, IMPL_BF16 = 0, 1, 2
 MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT = 0, 1, 2
 PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 3
+ABI_VERSION = 4
+STATIC_WS_BYTES = 16 << 20
 
 ERROR_NAMES = {
     -1: "FHOG_E_NULL", -2: "FHOG_E_SHAPE", -3: "FHOG_E_DTYPE", -4: "FHOG_E_STRIDE", -5: "FHOG_E_ALIGN",
@@ -79,6 +80,8 @@ def lib() -> ctypes.CDLL:
     L.fhog_select_impl.argtypes = [POINTER(BwdBwdArgs)]
     L.fhog_bwdbwd.restype = c_int
     L.fhog_bwdbwd.argtypes = [POINTER(BwdBwdArgs), c_void_p]
+    L.fhog_bwdbwd_static_ws.restype = c_int
+    L.fhog_bwdbwd_static_ws.argtypes = [POINTER(BwdBwdArgs), c_void_p]
     L.fhog_bwdbwd_pass.restype = c_int
     L.fhog_bwdbwd_pass.argtypes = [POINTER(BwdBwdArgs), c_int, c_void_p]
     L.fhog_last_error.restype = c_char_p

@@ -232,9 +232,15 @@ class BwdBwdPlan:
         _lib.check(self.lib.fhog_validate(ctypes.byref(self.args)))
         self.impl = self.lib.fhog_select_impl(ctypes.byref(self.args))
 
-    def run(self, stream: Optional[int] = None, only_pass: Optional[int] = None):
+    def run(self, stream: Optional[int] = None, only_pass: Optional[int] = None, static_ws: bool = False):
+        """Enqueue the call. ``static_ws``: through ``fhog_bwdbwd_static_ws``, which keeps the row statistics and partial
+        results in the library's own device array instead of this plan's workspace (``self.ws`` is then not written)."""
         s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream if stream is None else stream)
-        if only_pass is None:
+        if static_ws:
+            if only_pass is not None:
+                raise ValueError("static_ws runs the whole chain")
+            _lib.check(self.lib.fhog_bwdbwd_static_ws(ctypes.byref(self.args), s))
+        elif only_pass is None:
             _lib.check(self.lib.fhog_bwdbwd(ctypes.byref(self.args), s))
         else:
             _lib.check(self.lib.fhog_bwdbwd_pass(ctypes.byref(self.args), int(only_pass), s))

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FHOG_ABI_VERSION 3
+#define FHOG_ABI_VERSION 4
 
 /* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
 #define FHOG_DTYPE_BF16 0
@@ -141,6 +141,19 @@ int fhog_select_impl(const fhog_bwdbwd_args* args);
    schedule = FHOG_SCHEDULE_FUSED_STATS, dd and b come from one sweep (FHOG_PASS_DD_B) instead.
    Drop-in for the two launches + reduction of flash_bwdbwd (fhog/triton_bwdbwd.py:580-646). */
 int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
+
+/* fhog_bwdbwd for callers that cannot allocate device memory (code under HIP-graph capture, tight serving loops,
+   harnesses that forbid hipMalloc): the same passes, with the workspace (d | dd | b and the partial results of split
+   launches) in a device array of FHOG_STATIC_WS_BYTES that is part of the loaded library, one copy per GPU, held until
+   the process ends. args->ws and args->ws_bytes are not read; inputs and outputs stay the caller's. It has no
+   counterpart in the reference, which allocates D, dD and B with torch on every call (fhog/triton_bwdbwd.py:580-584).
+   Limits: batch * n_q <= FHOG_STATIC_WS_BYTES / 12 rows (FHOG_E_SHAPE beyond); launches split only as far as the array
+   has room. Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (two streams, two
+   threads) race on it; calls ordered on one stream do not. Nothing in the array has to start at zero: every word a
+   pass reads was written earlier in the same call. The first call on a device looks the array's address up
+   (hipGetSymbolAddress); no call allocates, frees or synchronises. */
+#define FHOG_STATIC_WS_BYTES (16 << 20)
+int fhog_bwdbwd_static_ws(const fhog_bwdbwd_args* args, void* hip_stream);
 
 /* One pass only (FHOG_PASS_*), for per-pass tests and profiling. Passes read the
    workspace rows written by earlier passes (stage 2 of the reference reads dD, B, D the

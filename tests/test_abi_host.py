@@ -34,7 +34,7 @@ def test_header_symbols_exported(L):
     assert set(names) >= {"fhog_abi_version", "fhog_bwdbwd_args_size", "fhog_bwdbwd_workspace_bytes", "fhog_validate", "fhog_select_impl",
                           "fhog_bwdbwd", "fhog_bwdbwd_pass", "fhog_last_error",
                           "fhog_attn_args_size", "fhog_attn_validate", "fhog_attn_fwd", "fhog_attn_bwd",
-                          "fhog_probe_mfma_rate", "fhog_bwdbwd_workspace_hint"}
+                          "fhog_probe_mfma_rate", "fhog_bwdbwd_workspace_hint", "fhog_bwdbwd_static_ws"}
     for n in names:
         assert hasattr(L, n), n
 
@@ -103,7 +103,7 @@ def test_attn_validate(L, mutate, backward, code, word):
 
 
 def test_version_and_workspace(L):
-    assert L.fhog_abi_version() == 3
+    assert L.fhog_abi_version() == 4
     assert L.fhog_bwdbwd_workspace_bytes(32, 4096) == 3 * 32 * 4096 * 4
     assert L.fhog_bwdbwd_workspace_bytes(-1, 5) == 0
 
