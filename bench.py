@@ -32,16 +32,25 @@ PASS_NAMES = {0: "rowdot_kernel (not in the 16-bit chain: its pass 1 writes d to
 PASS_CONTRACTIONS = {0: 0, 1: 3, 2: 5, 3: 9, 4: 8, 5: 5}
 
 
-def event_time_ms(fn, iters):
+def event_times_ms(fn, iters):
+    """Time `iters` calls of fn on torch's current stream (the stream the library's kernels are launched on), one event
+    between every two calls. Returns mean (first event to last: exactly `iters` calls between two synchronisations),
+    median and minimum of the per-call intervals, as the reference's do_bench reports them (fhog/benchhhh.py:58,76)."""
+    import statistics
     import torch
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
     torch.cuda.synchronize()
-    e0.record()
-    for _ in range(iters):
+    ev[0].record()
+    for i in range(iters):
         fn()
-    e1.record()
+        ev[i + 1].record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    each = [ev[i].elapsed_time(ev[i + 1]) for i in range(iters)]
+    return {"mean": ev[0].elapsed_time(ev[iters]) / iters, "median": statistics.median(each), "min": min(each)}
+
+
+def event_time_ms(fn, iters):
+    return event_times_ms(fn, iters)["mean"]
 
 
 def mfma_sustained(dev):
@@ -102,6 +111,28 @@ def first_order(w, x, iters):
             "note": "fhog_attn_fwd / fhog_attn_bwd including output allocation; not part of `value`"}
 
 
+def reference_sweep(max_n=65536):
+    """The first sizes of the reference's own benchmark sweep (fhog/benchhhh.py:15-27,93-110: one head, d = 64, fp16,
+    non-causal, N = 8192, 16384, ...; the x axis of assets/speedup.png): ms per call (median, min) and algorithmic
+    TFLOP/s. The whole list, up to N = 2097152, is `python flash-hob_amd/fhog/sweep.py`."""
+    import torch
+    from fhog.sweep import SIZES, sweep_point
+    return {"dtype": "f16", "d": 64, "heads": 1, "causal": False,
+            "points": [sweep_point(n, torch.float16, budget_ms=150.0, max_calls=30, min_calls=5) for n in SIZES if n <= max_n]}
+
+
+def traffic_bytes(workload, pass_id):
+    """HBM bytes per launch of one pass from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised under
+    profiles/ (the summary carries them in a machine-readable comment, written by fhog/rocprof_summary.py);
+    None when that workload or pass has no measurement."""
+    import re
+    for f in sorted((ROOT / "profiles").glob(f"bwdbwd_kernels_{workload}*.md")):
+        m = re.search(r"<!-- traffic_bytes: (\{.*?\}) -->", f.read_text())
+        if m:
+            return json.loads(m.group(1)).get(str(pass_id))
+    return None
+
+
 def cpu_baseline(w, x_cpu, heads, repeats):
     """torch autograd double-backward (fp32, materialised, one head at a time) on the host cores."""
     import torch
@@ -156,7 +187,8 @@ def main():
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     base_mem = torch.cuda.memory_allocated()
-    ms = event_time_ms(call, args.steps)
+    t_call = event_times_ms(call, args.steps)
+    ms = t_call["mean"]
     peak_extra = torch.cuda.max_memory_allocated() - base_mem
     peak_total = torch.cuda.max_memory_allocated()
     if args.profile_only:
@@ -175,8 +207,10 @@ def main():
         torch.cuda.synchronize()
         return
 
-    ms_plan = event_time_ms(plan.run, args.steps)
-    per_pass = {i: event_time_ms(lambda i=i: plan.run(only_pass=i), args.steps) for i in PASS_NAMES}
+    t_plan = event_times_ms(plan.run, args.steps)
+    ms_plan = t_plan["mean"]
+    t_pass = {i: event_times_ms(lambda i=i: plan.run(only_pass=i), args.steps) for i in PASS_NAMES}
+    per_pass = {i: t["mean"] for i, t in t_pass.items()}
     dom = max((i for i in per_pass if i != 5), key=PASS_CONTRACTIONS.get)   # the kernel with the largest share of the work
     plan_fused = fhog.BwdBwdPlan(x["Q"], x["K"], x["V"], o, x["dO"], x["ddQ"], x["ddK"], x["ddV"], L, w.scale,
                                  causal=w.causal, fused_stats=True)
@@ -193,6 +227,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms, 4),
+        "ms_per_step_median": round(t_call["median"], 4),
+        "ms_per_step_min": round(t_call["min"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -205,17 +241,21 @@ def main():
         "peak_mem_gb": round(peak_total / 1e9, 4),
         "peak_mem_call_gb": round(peak_extra / 1e9, 4),
         "ms_per_step_no_alloc": round(ms_plan, 4),
+        "ms_per_step_no_alloc_median": round(t_plan["median"], 4),
+        "ms_per_step_no_alloc_min": round(t_plan["min"], 4),
         "fused_stats_schedule": {"ms_per_step_no_alloc": round(ms_fused, 4),
                                  "value": round(w.flops_algorithmic / ms_fused / 1e9, 2),
                                  "note": "opt-in: dd and b from one sweep (22 recomputed products instead of 25)"},
         "ms_per_pass": {PASS_NAMES[i]: round(t, 4) for i, t in per_pass.items()},
+        "ms_per_pass_median_min": {PASS_NAMES[i]: [round(t["median"], 4), round(t["min"], 4)] for i, t in t_pass.items()},
         "roofline": {"bound": "mfma", "kernel": PASS_NAMES[dom], "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4),
                      "flops_per_launch": dom_flops, "ms_per_launch": round(per_pass[dom], 4),
-                     "traffic": TRAFFIC_BYTES.get((w.name, dom))},
+                     "ms_per_launch_median": round(t_pass[dom]["median"], 4), "traffic": traffic_bytes(w.name, dom)},
     }
     if not args.workload:
         out["other_workloads"] = other_workloads(dev, skip=w.name)
+        out["reference_sweep"] = reference_sweep()
     fo = first_order(w, x, min(args.steps, 20))
     if fo:
         out["first_order"] = fo
@@ -225,11 +265,6 @@ def main():
         out["cpu_baseline"] = cpu_baseline(w, x_cpu, min(args.cpu_heads, w.batch), repeats=2)
     print(json.dumps(out))
 
-
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), keyed by (workload, pass). None until measured for that kernel.
-TRAFFIC_BYTES = {("cfg2_bf16_causal_4096_d128", 3): int((510.1 + 64.4) * 2 ** 20),
-                 ("cfg2_bf16_causal_4096_d128", 4): int((372.1 + 64.0) * 2 ** 20)}
 
 if __name__ == "__main__":
     main()

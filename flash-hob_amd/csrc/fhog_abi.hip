@@ -3,6 +3,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
@@ -129,6 +130,8 @@ fhog::Params to_params(const fhog_bwdbwd_args* a) {
   mask_params(a->causal, a->window, a->n_q, a->n_k, &p.mask_off, &p.window);
   p.n_split = 1;
   p.part = nullptr;
+  const int order = fhog::tuning().order;
+  p.tile_major = order < 0 ? p.causal : order;
   return p;
 }
 
@@ -148,6 +151,7 @@ int wanted_split(const fhog_bwdbwd_args* a, int impl, int pass) {
   const int64_t groups = ((kside ? a->n_k : a->n_q) + 127) / 128 * a->batch;
   const int64_t streamed = ((kside ? a->n_q : a->n_k) + 31) / 32;
   int s = 1;
+  if (!fhog::tuning().split) return s;
   while (groups * s < 512 && s < 16 && streamed / (2 * s) >= 8) s *= 2;
   return s;
 }
@@ -253,6 +257,30 @@ int scratch_on_device(void** out) {
 }
 
 }  // namespace
+
+namespace fhog {
+const Tuning& tuning() {
+  static const Tuning t = [] {
+    Tuning r;
+    const char* env = getenv("FHOG_TUNE");
+    if (!env) return r;
+    char buf[256];
+    strncpy(buf, env, sizeof(buf) - 1);
+    buf[sizeof(buf) - 1] = 0;
+    for (char* tok = strtok(buf, ","); tok; tok = strtok(nullptr, ",")) {
+      char* eq = strchr(tok, '=');
+      if (!eq) continue;
+      *eq = 0;
+      const char* val = eq + 1;
+      if (!strcmp(tok, "b8")) r.b8 = atoi(val) != 0;
+      else if (!strcmp(tok, "order")) r.order = !strcmp(val, "tile") ? 1 : !strcmp(val, "slice") ? 0 : -1;
+      else if (!strcmp(tok, "split")) r.split = atoi(val) != 0;
+    }
+    return r;
+  }();
+  return t;
+}
+}  // namespace fhog
 
 extern "C" {
 

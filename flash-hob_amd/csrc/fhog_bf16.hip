@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
 
   // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
   int bh, tile, split = 0;
-  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch * p.n_split, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch * p.n_split, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
   if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
@@ -379,7 +379,7 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   constexpr int STAGE = 3 * TILE + STAT;   // Q, ddQ, dO tiles, statistics
 
   int bh, tile, split = 0;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, p.tile_major, bh, tile)) return;
   if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -604,7 +604,8 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   // three workgroups per CU), d = 64 (measured slower or equal) and small launches keep 128 rows.
   const unsigned g8 = grid_blocks((p.n_q + 255) / 256, slices);
   if constexpr (D == 128) {
-    if (!split && g8 >= 512 && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
+    const int b8 = tuning().b8;
+    if (!split && (b8 < 0 ? g8 >= 512 : b8 == 1) && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
       if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
       return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
     }

@@ -141,7 +141,7 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
 
   // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
   int bh, tile, split = 0;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
   if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
   constexpr int NC = D / 32;
 
   int bh, tile, split = 0;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split, false, p.tile_major, bh, tile)) return;
   if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars

@@ -181,8 +181,13 @@ struct Dma {
   // the register in between (clang warns about any reserved register on a clobber list; the warning is switched off here).
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-  __device__ __forceinline__ static void issue_one(uint32_t lds, uint32_t off, const __bf16* src) {
+  __device__ __forceinline__ static void issue_one(uint32_t lds, uint32_t off, const __bf16* src_) {
     const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds);
+    // the base address is wave-uniform; say so, or the "s" operand may be handed a vector register pair
+    // (the builtin returns a signed int: the halves are kept unsigned)
+    const uint64_t a = (uint64_t)src_;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    const __bf16* src = (const __bf16*)(((uint64_t)hi << 32) | lo);
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\t" ::"s"(m0), "v"(off), "s"(src) : "memory", "m0");
   }
 #pragma clang diagnostic pop

@@ -47,7 +47,21 @@ struct Params {
   // both head dims).
   int32_t n_split;
   float* part;
+  // Workgroup ids of one XCD enumerate its tiles (decode_block). tile_major: the slices that share the XCD advance
+  // through their tiles together instead of one slice after the other (the default with a mask).
+  int32_t tile_major;
 };
+
+// Launch choices that can be overridden for experiments through the environment variable FHOG_TUNE, a comma-separated
+// list of key=value (read once, on the host, at the first launch; never in a timed path):
+//   b8=0|1             b / dd+b sweeps at d = 128: 128-row workgroups of 4 waves | 256-row workgroups of 8 waves
+//                      (default: 8 waves when that still gives 512 workgroups)
+//   order=slice|tile   workgroup order within an XCD (default: tile-major with a mask, slice after slice without)
+//   split=0|1          let small launches split their streamed side (default 1)
+struct Tuning {
+  int b8 = -1, order = -1, split = 1;
+};
+const Tuning& tuning();
 
 // Kernel-side view of fhog_attn_args (first-order forward and backward).
 struct AttnParams {

@@ -41,15 +41,17 @@ def run_fhog(x, scale, causal, impl=None, **kw):
                              causal=causal, impl=impl, **kw)
 
 
-def reference_fp32_gpu(x, scale, causal, heads=None, head_chunk=1):
+def reference_fp32_gpu(x, scale, causal, heads=None, head_chunk=1, window=None):
     """fp32 torch autograd double-backward on materialised attention, on the GPU, head-chunked."""
     sel = (lambda t: t) if heads is None else (lambda t: t[heads])
     return autograd_double_backward(sel(x["Q"]), sel(x["K"]), sel(x["V"]), sel(x["dO"]), sel(x["ddQ"]), sel(x["ddK"]),
-                                    sel(x["ddV"]), scale, causal, dtype=torch.float32, head_chunk=head_chunk)
+                                    sel(x["ddV"]), scale, causal, dtype=torch.float32, head_chunk=head_chunk, window=window)
 
 
-def reference_fp64_cpu(x, scale, causal, window=None):
-    c = {n: t.detach().double().cpu().numpy() for n, t in x.items()}
+def reference_fp64_cpu(x, scale, causal, window=None, heads=None):
+    """fp64 closed form on the CPU (outputs and the row vectors d, dd, b), optionally on a few (batch*head) slices."""
+    sel = (lambda t: t) if heads is None else (lambda t: t[heads])
+    c = {n: sel(t).detach().double().cpu().numpy() for n, t in x.items()}
     return closed_form(c["Q"], c["K"], c["V"], c["dO"], c["ddQ"], c["ddK"], c["ddV"], scale, causal, window=window)
 
 

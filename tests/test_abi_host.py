@@ -170,6 +170,26 @@ def test_workspace_hint(L):
     assert L.fhog_bwdbwd_workspace_hint(ctypes.byref(a)) == 0   # invalid arguments
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_workspace_hint_stays_below_its_stated_bound(L, d):
+    """Whatever batch and N: the partial results of split launches take fewer than 2 * 131072 * d floats (a pass stops
+    doubling its split once it has 512 workgroups), so the workspace stays linear in N plus a constant."""
+    worst = 0
+    for batch in (1, 2, 3, 4, 5, 7, 8, 15, 16, 31, 32, 33, 64):
+        for n in [128 * k + r for k in (1, 2, 3, 5, 8, 13, 16, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 511, 512, 1023, 1024)
+                  for r in (-127, 0)]:
+            a = good_args()
+            a.batch, a.n_q, a.n_k, a.d = batch, n, n, d
+            a.stride_qn = a.stride_kn = d
+            a.stride_qb = a.stride_kb = n * d
+            hint = L.fhog_bwdbwd_workspace_hint(ctypes.byref(a))
+            stats = (3 * batch * n * 4 + 15) // 16 * 16
+            assert hint >= L.fhog_bwdbwd_workspace_bytes(batch, n)
+            worst = max(worst, hint - stats)
+    assert 0 < worst < 2 * 131072 * d * 4
+    assert worst > 2 * 65536 * d * 4      # the bound is not slack by a factor of two: some shape comes close
+
+
 def test_probe_rejects_bad_arguments(L):
     flops = ctypes.c_double()
     assert L.fhog_probe_mfma_rate(None, 256, 10, 0, ctypes.byref(flops), None) == -1

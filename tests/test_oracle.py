@@ -237,3 +237,28 @@ def test_band_mask_reductions_to_known_cases():
     np.testing.assert_allclose(one["dk2"], 0, atol=1e-12)
     np.testing.assert_allclose(one["dv2"], 0, atol=1e-12)
     np.testing.assert_allclose(one["ddo"], x["ddv"], atol=1e-12)   # O_i = V_i, so ddO_i = ddV_i
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(24, 24, 8), (33, 33, 16), (17, 40, 8)])
+def test_first_backward_and_forward_equal_sdpa_autograd(shape, causal):
+    """forward_o_lse and first_backward (the oracle of the first-order kernels and of the adjoint test) against a
+    library routine: torch's scaled_dot_product_attention and its autograd, in float64."""
+    n_q, n_k, d = shape
+    if causal and n_q != n_k:
+        pytest.skip("causal is defined for N_Q == N_K")
+    rng = np.random.default_rng(11)
+    x = rand_inputs(rng, n_q, n_k, d, batch=(2,))
+    scale = 0.37
+    q, k, v = (torch.tensor(x[n], dtype=torch.float64, requires_grad=True) for n in ("q", "k", "v"))
+    out = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=causal, scale=scale)
+    want = torch.autograd.grad(out, (q, k, v), torch.tensor(x["do"]))
+    o, lse = forward_o_lse(x["q"], x["k"], x["v"], scale, causal)
+    assert normalised_max_error(o, out.detach()) < 1e-12
+    s = scale * torch.einsum("bid,bjd->bij", q.detach(), k.detach())
+    if causal:
+        s = s.masked_fill(~torch.ones(n_q, n_k, dtype=torch.bool).tril(), float("-inf"))
+    assert normalised_max_error(lse, torch.logsumexp(s, -1)) < 1e-12
+    got = first_backward(x["q"], x["k"], x["v"], x["do"], scale, causal)
+    for name, a, b in zip(("dq", "dk", "dv"), got, want):
+        assert normalised_max_error(a, b) < 1e-12, name
