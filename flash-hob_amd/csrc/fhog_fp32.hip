@@ -3,9 +3,11 @@
 // MFMA cannot reach 1e-4) and d = 32; it takes bf16 and fp16 tensors of any shape too.
 // No atomics, nothing of shape (N_Q, N_K) leaves the chip.
 //
-// One kernel template for the four sweeps. A workgroup of 1, 2 or 4 wave64 owns 32 stationary
-// rows per wave (queries in passes 1-3, keys in pass 4) and keeps their operands in registers;
-// the other side streams through LDS in 32-row tiles shared by the waves. First-level products are
+// One kernel template for the four sweeps. A workgroup of 4 wave64 owns 32 stationary rows per wave
+// (queries in passes 1-3, keys in pass 4) and keeps their operands in registers; the other side
+// streams through LDS in 32-row tiles shared by the waves. Small launches (WS = 2 or 4) put WS waves
+// on the same 32 rows instead: each takes every WS-th streamed tile and the partial results are
+// added through LDS in a fixed order, so a short problem is spread over WS times the workgroups. First-level products are
 // computed with the streamed rows as M and the stationary rows as N, so a lane owns ONE stationary
 // row and its registers run over the streamed rows. Such an accumulator is, as it stands, the B
 // operand of the second-level products (contraction over the streamed rows; the A operand is read
@@ -188,7 +190,7 @@ __device__ inline void store_acc(T* dst, int64_t ld, int row, int n, const f32x1
 }
 
 // PASS 1: dd (Q-tiled), 2: b (Q-tiled), 3: dQ2 and ddO (Q-tiled), 4: dK2 and dV2 (K-tiled).
-template <typename T, int D, int PASS, bool MASKED>
+template <typename T, int D, int PASS, bool MASKED, int WS = 1>
 __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   constexpr bool KSIDE = PASS == 4;                          // the stationary rows are keys
@@ -198,9 +200,12 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   constexpr int NREG = LAST_IN_LDS ? 3 : NR;
   constexpr int J = D / 8, CB = D / 32, TF = Tile<D>::FLOATS;
 
-  constexpr int nw = 4, nthr = 64 * nw;   // waves per workgroup (waves without rows still help with the loads)
+  static_assert(WS == 1 || D <= 64, "wave split needs WS staged tiles per tensor in LDS");
+  constexpr int nthr = 256;        // 4 waves (waves without rows still help with the loads)
+  constexpr int nw = 4 / WS;       // groups of 32 stationary rows per workgroup, WS waves on each
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = wv / WS, ws = wv % WS;   // row group of the wave, and which of its streamed tiles it takes
   const int n = lane & 31, h = lane >> 5;
   const int n_sta = KSIDE ? p.n_k : p.n_q, n_str = KSIDE ? p.n_q : p.n_k;
   // All tiles of a slice on one XCD (one L2 streams the slice's other side). With a mask the work of a tile grows (or
@@ -217,9 +222,9 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   const T* str[4] = {(const T*)(KSIDE ? p.q : p.k) + (KSIDE ? qoff : koff), (const T*)(KSIDE ? p.ddq : p.ddk) + (KSIDE ? qoff : koff),
                      (const T*)(KSIDE ? p.dO : p.v) + (KSIDE ? qoff : koff), (const T*)p.ddv + koff};
 
-  float* tiles = smem;                           // NT streamed tiles
-  float* stat = tiles + NT * TF;                 // pass 4: L, d, dd, b of the 32 streamed queries
-  float* sta_lds = stat + (KSIDE ? 4 * TR : 0);  // pass 4, d = 128: ddV rows of each wave
+  float* tiles = smem;                                // WS stages of NT streamed tiles
+  float* stat = tiles + WS * NT * TF;                 // pass 4: L, d, dd, b of the 32 streamed queries of each stage
+  float* sta_lds = stat + (KSIDE ? WS * 4 * TR : 0);  // pass 4, d = 128: ddV rows of each wave
   const int64_t srow = (int64_t)bh * p.n_q;
 
 #pragma unroll 1
@@ -272,7 +277,7 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
   // Streaming: up to d = 64 the next tile is fetched into registers while this one is computed on and written to
   // LDS behind the step (PRE f32x4 per tensor and thread); at d = 128 the registers are taken and the tile is
   // loaded between two barriers.
-  constexpr bool PREFETCH = D <= 64;
+  constexpr bool PREFETCH = D <= 64 && WS == 1;
   constexpr int C4 = D / 4, PRE = PREFETCH ? TR * C4 / nthr : 1;
   f32x4_t pre[NT][PRE];
   float pre_stat = 0.f;
@@ -313,20 +318,28 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
     publish();
   }
 
-  for (int s0 = s_begin; s0 < s_end; s0 += TR) {
+  for (int sb = s_begin; sb < s_end; sb += WS * TR) {
     __syncthreads();
     if (PREFETCH) {
-      if (s0 + TR < s_end) fetch(s0 + TR);
+      if (sb + TR < s_end) fetch(sb + TR);
     } else {
-      load_tile_pair<T, D>(tiles, tiles + TF, str[0], str[1], str_ld, s0, n_str, tid);
-      if (NT > 2) load_tile_pair<T, D>(tiles + 2 * TF, tiles + (NT - 1) * TF, str[2], str[NT - 1], str_ld, s0, n_str, tid);
-      if (KSIDE && tid < 4 * TR) {
-        const int qi = s0 + (tid & 31);
-        stat[tid] = qi < p.n_q ? stat_src[qi] : 0.f;
+#pragma unroll
+      for (int g = 0; g < WS; g++) {   // stage g holds the tile of the waves with ws == g
+        float* tg = tiles + g * NT * TF;
+        load_tile_pair<T, D>(tg, tg + TF, str[0], str[1], str_ld, sb + g * TR, n_str, tid);
+        if (NT > 2) load_tile_pair<T, D>(tg + 2 * TF, tg + (NT - 1) * TF, str[2], str[NT - 1], str_ld, sb + g * TR, n_str, tid);
+        if (KSIDE && tid < 4 * TR) {
+          const int qi = sb + g * TR + (tid & 31);
+          stat[g * 4 * TR + tid] = qi < p.n_q ? stat_src[qi] : 0.f;
+        }
       }
       __syncthreads();
     }
+    const int s0 = sb + ws * TR;
+    const float* const tiles = smem + ws * NT * TF;
+    const float* const stat = smem + WS * NT * TF + ws * 4 * TR;
     [&]() {
+    if (WS > 1 && s0 >= s_end) return;   // the last round of tiles may be short
     // Every pair of this wave's rows with this tile hidden: nothing to add. Not at d = 128, where the extra loop
     // edge makes the register allocator spill; there the element mask alone zeroes the block.
     bool dead = false;
@@ -402,9 +415,40 @@ __global__ void __launch_bounds__(256) sweep_fp32(Params p) {
     }
     if (PASS >= 3) mma_second<D>(acc0, w, t0, lane);             // dQ2 += dS' K | dK2 += dS'^T Q
     }();
-    if (PREFETCH && s0 + TR < s_end) {
+    if (PREFETCH && sb + TR < s_end) {
       __syncthreads();   // every wave is done reading the tile
       publish();
+    }
+  }
+
+  if (WS > 1) {
+    // the WS waves of a row group add their partial results through LDS in the order of ws; the wave with ws == 0
+    // holds the sum and stores it
+    __syncthreads();   // the streamed tiles are no longer read
+    float* xch = smem + ((wave * (WS - 1) + (ws - 1)) * (PASS <= 2 ? 1 : 2 * CB * 16)) * 64 + lane;
+    if (ws > 0) {
+      if (PASS <= 2) {
+        xch[0] = red;
+      } else {
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) xch[(cb * 16 + r) * 64] = acc0[cb][r], xch[((CB + cb) * 16 + r) * 64] = acc1[cb][r];
+      }
+    }
+    __syncthreads();
+    if (ws > 0) continue;
+#pragma unroll
+    for (int o = 1; o < WS; o++) {
+      const float* src = smem + ((wave * (WS - 1) + (o - 1)) * (PASS <= 2 ? 1 : 2 * CB * 16)) * 64 + lane;
+      if (PASS <= 2) {
+        red += src[0];
+      } else {
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc0[cb][r] += src[(cb * 16 + r) * 64], acc1[cb][r] += src[((CB + cb) * 16 + r) * 64];
+      }
     }
   }
 
@@ -445,21 +489,36 @@ __global__ void __launch_bounds__(256) rowdot_kernel(Params p) {
   if (r < rows && sub == 0) p.ws_d[r] = acc;
 }
 
-template <typename T, int D, int PASS, bool MASKED>
-hipError_t launch_sweep(const Params& p, hipStream_t s) {
+template <typename T, int D, int PASS, bool MASKED, int WS>
+hipError_t launch_sweep_ws(const Params& p, hipStream_t s) {
   constexpr bool KSIDE = PASS == 4;
   constexpr int NT = PASS == 1 ? 2 : (KSIDE ? 3 : 4);
   const int64_t n_rows = KSIDE ? p.n_k : p.n_q;
-  constexpr int nw = 4;   // waves per workgroup: measured best at every size (the waves share the streamed tiles and their loads)
-  size_t floats = (size_t)NT * Tile<D>::FLOATS + (KSIDE ? 4 * TR : 0);
+  constexpr int nw = 4 / WS;   // 32-row groups per workgroup
+  size_t floats = (size_t)WS * NT * Tile<D>::FLOATS + (KSIDE ? WS * 4 * TR : 0);
   if (KSIDE && D == 128) floats += (size_t)nw * Tile<D>::FLOATS;
   const int smem = (int)(floats * sizeof(float));
   const int n_tiles = (int)((n_rows + TR * nw - 1) / (TR * nw));
-  const dim3 grid(bf16k::grid_blocks(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch)), block(64 * nw);
-  const hipError_t e = hipFuncSetAttribute((const void*)sweep_fp32<T, D, PASS, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  const dim3 grid(bf16k::grid_blocks(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch)), block(256);
+  const hipError_t e = hipFuncSetAttribute((const void*)sweep_fp32<T, D, PASS, MASKED, WS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL((sweep_fp32<T, D, PASS, MASKED>), grid, block, smem, s, p);
+  hipLaunchKernelGGL((sweep_fp32<T, D, PASS, MASKED, WS>), grid, block, smem, s, p);
   return hipGetLastError();
+}
+
+// Four waves on 128 stationary rows is the best shape whenever that fills the GPU (the waves share the streamed tiles
+// and their loads). A launch with fewer than 128 such workgroups (256 CUs) puts two or four waves on the same 32 rows
+// instead (d <= 64: the stages of all waves have to fit the LDS): a 256-token problem of two heads is 4 workgroups
+// otherwise, each running its eight streamed tiles one after the other.
+template <typename T, int D, int PASS, bool MASKED>
+hipError_t launch_sweep(const Params& p, hipStream_t s) {
+  if constexpr (D <= 64) {
+    const int64_t n_rows = PASS == 4 ? p.n_k : p.n_q, n_str = PASS == 4 ? p.n_q : p.n_k;
+    const int64_t groups = (n_rows + 127) / 128 * p.batch / (MASKED ? 2 : 1);
+    if (groups < 64 && n_str > 2 * TR) return launch_sweep_ws<T, D, PASS, MASKED, 4>(p, s);
+    if (groups < 128 && n_str > TR) return launch_sweep_ws<T, D, PASS, MASKED, 2>(p, s);
+  }
+  return launch_sweep_ws<T, D, PASS, MASKED, 1>(p, s);
 }
 
 template <typename T, int D>

@@ -69,14 +69,41 @@ def counters(path):
     return {k: {c: sum(v) / len(v) for c, v in d.items()} for k, d in a.items()}
 
 
+def compare(w, variants):
+    """One table row per (variant, double-backward kernel): average duration, matrix-pipe occupancy, clock, HBM bytes read.
+    `variants`: list of (label, directory holding prof_kt, prof_fetch, prof_sq of a run made under that FHOG_TUNE)."""
+    P = print
+    P("| FHOG_TUNE | kernel | calls | avg ns | MFMA busy fraction | clock GHz | HBM read MiB | HBM read / algorithmic |")
+    P("|---|---|---|---|---|---|---|---|")
+    for label, root in variants:
+        root = Path(root)
+        kt = {short(r["Name"]): r for r in csv.DictReader(open(root / "prof_kt" / "kt_kernel_stats.csv")) if "fhog" in r["Name"]}
+        fe = counters(root / "prof_fetch" / "f_counter_collection.csv")
+        sq = counters(root / "prof_sq" / "s_counter_collection.csv")
+        sf = 262144 / fe["calib"]["FETCH_SIZE"]
+        for k in sorted(kt, key=lambda k: str(pass_of(k))):
+            p = pass_of(k)
+            if not isinstance(p, int) or p == 0 or k not in sq or int(kt[k]["Calls"]) < 4:
+                continue
+            d = sq[k]
+            cyc, ns = d["SQ_BUSY_CYCLES"] / 32, float(kt[k]["AverageNs"])
+            f = fe[k]["FETCH_SIZE"] * sf / 1024
+            P(f"| {label} | {k} | {kt[k]['Calls']} | {ns:.0f} | {d['SQ_VALU_MFMA_BUSY_CYCLES'] / 1024 / cyc:.3f} | {cyc / ns:.2f} | {f:.1f} | "
+              f"{f / algorithmic_mib(w, p)[0]:.2f} |")
+
+
 def main():
     from fhog.workloads import WORKLOADS
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", required=True)
     ap.add_argument("--root", default="gpurun_out", help="directory holding prof_kt, prof_fetch, prof_write, prof_sq")
     ap.add_argument("--note", default="", help="free text appended to the summary")
+    ap.add_argument("--compare", nargs="+", metavar="LABEL@DIR", help="instead of a summary: one table over runs made under "
+                    "different FHOG_TUNE settings (each DIR holds prof_kt, prof_fetch, prof_sq)")
     args = ap.parse_args()
     w = WORKLOADS[args.workload]
+    if args.compare:
+        return compare(w, [tuple(c.rsplit("@", 1)) for c in args.compare])
     root = Path(args.root)
     kt = {short(r["Name"]): r for r in csv.DictReader(open(root / "prof_kt" / "kt_kernel_stats.csv")) if "fhog" in r["Name"]}
     fe = counters(root / "prof_fetch" / "f_counter_collection.csv")

@@ -96,6 +96,26 @@ def test_fp32_family_ragged(shape, causal, dtype):
         assert normalised_max_error(got, ref[name]) < stat_tol, name
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 256, 256, 64), (70, 128, 200, 32), (130, 128, 96, 64), (40, 300, 300, 64), (3, 100, 40, 64)])
+def test_fp32_family_launch_sizes(shape, causal):
+    """The fp32-MFMA kernels put one, two or four waves on the same 32 stationary rows depending on how many workgroups
+    the launch has (four, each taking every fourth streamed tile, for a problem as small as the first benchmark
+    configuration): every regime against the fp64 closed form at the fp32 gate, row statistics included."""
+    batch, n_q, n_k, d = shape
+    if causal:
+        n_k = n_q
+    x = make_case(batch, n_q, n_k, d, torch.float32, seed=27)
+    scale = d ** -0.5
+    x = with_caches(x, scale, causal)
+    outs = run_fhog(x, scale, causal, return_stats=True)
+    ref = reference_fp64_cpu(x, scale, causal)
+    e = errors(outs[:4], [ref[n] for n in NAMES])
+    assert max(e.values()) < 1e-4, e
+    for got, name in zip(outs[4], ("d", "dd", "b")):
+        assert normalised_max_error(got, ref[name]) < 1e-4, name
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("mask", [("bottom_right", None, 100, 177), ("bottom_right", 40, 100, 177), (True, 33, 160, 160),
                                   ("bottom_right", 1, 64, 96), ("bottom_right", 500, 31, 31), (True, 7, 256, 256)])
