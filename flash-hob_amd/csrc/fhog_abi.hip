@@ -187,6 +187,10 @@ int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& base, int impl, int 
   return FHOG_OK;
 }
 
+// bf16 / fp16 tensors with d in {64, 128} run on the 16-bit MFMA kernels, everything else (fp32 tensors, d = 32) on the
+// fp32-MFMA ones
+bool attn_on_16bit_kernels(const fhog_attn_args* a) { return a->dtype != FHOG_DTYPE_FP32 && (a->d == 64 || a->d == 128); }
+
 int validate_attn(const fhog_attn_args* a, int backward) {
   if (!a) return fail(FHOG_E_NULL, "args is NULL");
   const void* ptrs[] = {a->q, a->k, a->v, a->o, a->lse, a->dO, a->dq, a->dk, a->dv, a->ws};
@@ -196,20 +200,22 @@ int validate_attn(const fhog_attn_args* a, int backward) {
     if (!ptrs[i]) return fail(FHOG_E_NULL, "pointer '%s' is NULL", names[i]);
     if (!aligned16(ptrs[i])) return fail(FHOG_E_ALIGN, "pointer '%s' is not 16-byte aligned", names[i]);
   }
-  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP16)
-    return fail(FHOG_E_DTYPE, "the first-order kernels take bf16 or fp16 tensors (dtype %d given)", a->dtype);
+  if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP16 && a->dtype != FHOG_DTYPE_FP32)
+    return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
   if (a->batch < 1 || a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld outside 1..65535", (long long)a->batch);
   if (a->n_q < 1 || a->n_k < 1 || a->n_q > (1 << 24) || a->n_k > (1 << 24) || a->batch * a->n_q >= (int64_t)1 << 31)
     return fail(FHOG_E_SHAPE, "n_q/n_k out of range");
   if (const int rc = check_mask(a->causal, a->window, a->n_q, a->n_k)) return rc;
-  if (!fhog::bf16_shape_supported(a->n_q, a->n_k, a->d, a->causal))
-    return fail(FHOG_E_SHAPE, "the first-order kernels need d in {64,128}");
-  // the forward takes the running maximum of the raw scores and scales it afterwards, which needs scale > 0
-  if (!isfinite(a->scale) || a->scale <= 0.f) return fail(FHOG_E_SCALE, "scale must be finite and positive (got %g)", (double)a->scale);
+  if (a->d != 32 && a->d != 64 && a->d != 128) return fail(FHOG_E_SHAPE, "head dim %lld not in {32, 64, 128}", (long long)a->d);
+  if (!isfinite(a->scale)) return fail(FHOG_E_SCALE, "scale is not finite");
+  // the 16-bit forward takes the running maximum of the raw scores and scales it afterwards, which needs scale > 0
+  if (attn_on_16bit_kernels(a) && a->scale <= 0.f)
+    return fail(FHOG_E_SCALE, "the 16-bit kernels need a positive scale (got %g)", (double)a->scale);
+  const int vec = a->dtype == FHOG_DTYPE_FP32 ? 4 : 8;  // elements per 16 bytes
   if (a->stride_qn < a->d || a->stride_kn < a->d) return fail(FHOG_E_STRIDE, "row stride smaller than d");
   if (a->stride_qn > kMaxRowStride || a->stride_kn > kMaxRowStride) return fail(FHOG_E_STRIDE, "row stride above 2^24 elements");
-  if (a->stride_qn % 8 || a->stride_kn % 8 || a->stride_qb % 8 || a->stride_kb % 8)
-    return fail(FHOG_E_STRIDE, "strides must be multiples of 8 elements (16 bytes)");
+  if (a->stride_qn % vec || a->stride_kn % vec || a->stride_qb % vec || a->stride_kb % vec)
+    return fail(FHOG_E_STRIDE, "strides must be multiples of %d elements (16 bytes)", vec);
   if (a->batch > 1 && (a->stride_qb < a->n_q * a->stride_qn || a->stride_kb < a->n_k * a->stride_kn))
     return fail(FHOG_E_STRIDE, "batch stride smaller than one (n, d) slice");
   return FHOG_OK;
@@ -297,7 +303,8 @@ int fhog_attn_validate(const fhog_attn_args* args, int backward) { return valida
 int fhog_attn_fwd(const fhog_attn_args* args, void* hip_stream) {
   const int rc = validate_attn(args, 0);
   if (rc != FHOG_OK) return rc;
-  const hipError_t e = fhog::launch_attn_bf16(to_attn_params(args), 0, (hipStream_t)hip_stream);
+  const hipError_t e = attn_on_16bit_kernels(args) ? fhog::launch_attn_bf16(to_attn_params(args), 0, (hipStream_t)hip_stream)
+                                                   : fhog::launch_attn_fp32(to_attn_params(args), args->dtype, 0, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "attention forward: HIP error %d (%s)", (int)e, hipGetErrorString(e));
   return FHOG_OK;
 }
@@ -316,7 +323,9 @@ int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream) {
   rd.n_q = p.n_q;
   rd.d = p.d;
   hipError_t e = fhog::launch_rowdot(rd, args->dtype, (hipStream_t)hip_stream);
-  for (int which = 1; which <= 2 && e == hipSuccess; which++) e = fhog::launch_attn_bf16(p, which, (hipStream_t)hip_stream);
+  for (int which = 1; which <= 2 && e == hipSuccess; which++)
+    e = attn_on_16bit_kernels(args) ? fhog::launch_attn_bf16(p, which, (hipStream_t)hip_stream)
+                                    : fhog::launch_attn_fp32(p, args->dtype, which, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "attention backward: HIP error %d (%s)", (int)e, hipGetErrorString(e));
   return FHOG_OK;
 }

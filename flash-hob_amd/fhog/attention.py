@@ -10,10 +10,11 @@ commented stub (``fhog/triton_bwdbwd.py:538-554``).  Here it is wired:
     AttnBwd.forward          -> dQ, dK, dV   (first-order backward)
     AttnBwd.backward         -> flash_bwdbwd(...) -> dQ', dK', dV', ddO
 
-The forward and the first-order backward are the callers on either side of the hot path.  For bf16 and fp16
-tensors with d in {64, 128} they run as HIP kernels of
-the same library (``fhog_attn_fwd`` / ``fhog_attn_bwd``); every other dtype or shape takes
-linear-memory torch compositions on the GPU (blocked over heads and query rows, fp32 accumulation).
+The forward and the first-order backward are the callers on either side of the hot path.  They run as HIP
+kernels of the same library (``fhog_attn_fwd`` / ``fhog_attn_bwd``): 16-bit MFMA kernels for bf16 and fp16 tensors
+with d in {64, 128}, fp32-MFMA kernels for fp32 tensors and d = 32.  A linear-memory torch composition on the GPU
+(blocked over heads and query rows, fp32 accumulation) remains for arguments the kernels reject (a non-positive
+scale on 16-bit tensors) and as the second implementation the tests compare with (``use_hip=False``).
 The double-backward is always the HIP library.
 """
 from __future__ import annotations
@@ -28,7 +29,7 @@ import torch
 from . import _lib
 from .bwdbwd import flash_bwdbwd, mask_code
 
-_HIP_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16}
+_HIP_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_FP16, torch.float32: _lib.DTYPE_FP32}
 _BLOCK_ELEMS = 1 << 26  # fp32 elements of one materialised (heads, rows, N_K) block (256 MiB)
 
 
@@ -146,7 +147,8 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, w
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16/fp16, d in {64,128}, GPU)")
+            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16, fp16 or fp32 on the GPU, d in {32, 64, 128}, "
+                             "a positive scale for 16-bit tensors)")
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
@@ -175,7 +177,8 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal, *, window: Optio
         if res is not None:
             return res
         if use_hip:
-            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16/fp16, d in {64,128}, GPU)")
+            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16, fp16 or fp32 on the GPU, d in {32, 64, 128}, "
+                             "a positive scale for 16-bit tensors)")
     dq = torch.empty_like(q)
     dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)

@@ -161,8 +161,9 @@ int fhog_bwdbwd_static_ws(const fhog_bwdbwd_args* args, void* hip_stream);
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream);
 
 /* ---- first-order attention: the callers on either side of the double-backward ---------------------------
- * bf16 or fp16 tensors, d in {64, 128}, any n_q and n_k (fhog_attn_validate tells); the layout rules
- * above apply. O and dO/dQ share the q strides, dK/dV the k strides. */
+ * bf16, fp16 or fp32 tensors, d in {32, 64, 128}, any n_q and n_k (fhog_attn_validate tells); the layout rules
+ * above apply. bf16 / fp16 tensors with d in {64, 128} run on 16-bit MFMA kernels (they need scale > 0), fp32
+ * tensors and d = 32 on fp32-MFMA kernels. O and dO/dQ share the q strides, dK/dV the k strides. */
 typedef struct fhog_attn_args {
   const void* q;   /* (batch, n_q, d) */
   const void* k;   /* (batch, n_k, d) */
@@ -177,7 +178,7 @@ typedef struct fhog_attn_args {
   int64_t batch, n_q, n_k, d;
   int64_t stride_qb, stride_qn, stride_kb, stride_kn;
   float scale;
-  int32_t dtype;   /* FHOG_DTYPE_BF16 | FHOG_DTYPE_FP16 */
+  int32_t dtype;   /* FHOG_DTYPE_* */
   int32_t causal;  /* FHOG_MASK_*, as in fhog_bwdbwd_args */
   int32_t window;  /* sliding window length in keys, 0 = none; needs a causal mask */
 } fhog_attn_args;

@@ -78,9 +78,13 @@ def good_attn_args():
     (lambda a: setattr(a, "dO", 0), 0, 0, ""),            # forward does not look at the backward-only pointers
     (lambda a: setattr(a, "dO", 0), 1, -1, "dO"),
     (lambda a: setattr(a, "lse", 0), 0, -1, "lse"),
-    (lambda a: setattr(a, "dtype", 1), 0, -3, "bf16"),
+    (lambda a: setattr(a, "dtype", 1), 0, 0, ""),             # fp32 tensors: the fp32-MFMA first-order kernels
+    (lambda a: setattr(a, "dtype", 5), 0, -3, "dtype"),
+    (lambda a: (setattr(a, "dtype", 1), setattr(a, "stride_kn", 68), setattr(a, "stride_kb", 512 * 68)), 1, 0, ""),   # 16 bytes = 4 floats
+    (lambda a: (setattr(a, "dtype", 1), setattr(a, "scale", -0.125)), 0, 0, ""),   # any sign of the scale there
+    (lambda a: setattr(a, "d", 32), 1, 0, ""),                # d = 32 as well
+    (lambda a: setattr(a, "d", 96), 0, -2, "head dim"),
     (lambda a: setattr(a, "n_q", 200), 0, 0, ""),           # ragged lengths are fine
-    (lambda a: setattr(a, "d", 32), 0, -2, "d in"),
     (lambda a: setattr(a, "causal", 1), 0, -6, "causal"),   # top-left needs n_q == n_k
     (lambda a: setattr(a, "causal", 2), 0, 0, ""),
     (lambda a: (setattr(a, "causal", 2), setattr(a, "window", 17)), 1, 0, ""),

@@ -127,17 +127,78 @@ def test_strided_rows_and_4d_input():
     assert torch.equal(o4.flatten(0, 1), o) and torch.equal(L4.flatten(0, 1), L)
 
 
-def test_unsupported_arguments_take_the_torch_composition_or_raise():
+@pytest.mark.parametrize("causal", [False, True, "bottom_right"])
+@pytest.mark.parametrize("case", [(torch.float32, 2, 256, 256, 64), (torch.float32, 3, 100, 177, 128), (torch.float32, 2, 33, 129, 32),
+                                  (torch.bfloat16, 2, 200, 200, 32), (torch.float16, 1, 300, 300, 32), (torch.float32, 1, 1, 1, 64)])
+def test_fp32_mfma_first_order_kernels(case, causal):
+    """fp32 tensors (the producer of O and L for the first benchmark configuration) and d = 32 run on the fp32-MFMA
+    first-order kernels: O, L, dQ, dK, dV against the fp64 oracle, at the fp32 gate for fp32 tensors."""
     import fhog
-    x = make_case(2, 200, 200, 32, torch.bfloat16, seed=24)   # d = 32 is not covered by the HIP first-order kernels
+    from fhog.attention import attention_backward
+    dtype, batch, n_q, n_k, d = case
+    window = None
+    if causal is True:
+        n_k = n_q
+    elif causal == "bottom_right":
+        n_k, window = max(n_k, n_q), 40
+    x = make_case(batch, n_q, n_k, d, dtype, seed=29)
+    scale = d ** -0.5
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], scale, causal, window=window, use_hip=True)
+    o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), scale, causal, window)
+    tol = 1e-4 if dtype == torch.float32 else 1e-2
+    assert o.dtype == dtype and L.dtype == torch.float32
+    assert normalised_max_error(o, o_ref) < tol
+    assert (L.double().cpu() - torch.from_numpy(l_ref)).abs().max() < (1e-4 if dtype == torch.float32 else 2e-3)
+    got = attention_backward(x["Q"], x["K"], x["V"], o, x["dO"], L, scale, causal, window=window, use_hip=True)
+    ref = first_backward(_np(x["Q"]), _np(x["K"]), _np(x["V"]), _np(x["dO"]), scale, causal, window)
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        assert a.dtype == dtype
+        assert normalised_max_error(a, b) < (1e-4 if dtype == torch.float32 else 2e-2), name
+
+
+def test_fp32_kernels_take_a_negative_scale_and_16_bit_ones_fall_back():
+    """The fp32-MFMA forward scales the scores before it takes their maximum: any sign of the scale. The 16-bit forward
+    needs a positive one: use_hip=True raises, the default takes the torch composition."""
+    import fhog
+    y = make_case(2, 128, 160, 64, torch.float32, seed=24)
+    o, L = fhog.attention_forward(y["Q"], y["K"], y["V"], -0.2, False, use_hip=True)
+    o_ref, l_ref = forward_o_lse(_np(y["Q"]), _np(y["K"]), _np(y["V"]), -0.2, False)
+    assert normalised_max_error(o, o_ref) < 1e-4
+    assert (L.double().cpu() - torch.from_numpy(l_ref)).abs().max() < 1e-4
+    x = make_case(2, 128, 160, 64, torch.bfloat16, seed=24)
     with pytest.raises(ValueError):
-        fhog.attention_forward(x["Q"], x["K"], x["V"], 0.125, False, use_hip=True)
-    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], 0.125, False)
-    o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), 0.125, False)
+        fhog.attention_forward(x["Q"], x["K"], x["V"], -0.2, False, use_hip=True)
+    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], -0.2, False)
+    o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), -0.2, False)
     assert normalised_max_error(o, o_ref) < 1e-2
-    y = make_case(1, 128, 128, 64, torch.float32, seed=24)
-    with pytest.raises(ValueError):
-        fhog.attention_forward(y["Q"], y["K"], y["V"], 0.125, False, use_hip=True)
+
+
+def test_fp32_autograd_chain_runs_on_hip_kernels_only():
+    """attention() on fp32 tensors: forward, first backward and double-backward are all kernels of the library (the torch
+    composition is switched off for the duration of the test)."""
+    import sys
+    import fhog
+    A = sys.modules["fhog.attention"]   # the module (fhog.attention the attribute is the function of that name)
+    g = torch.Generator().manual_seed(30)
+    mk = lambda *s: torch.randn(*s, generator=g).cuda()
+    q, k, v, w = mk(2, 160, 64), mk(2, 160, 64), mk(2, 160, 64), mk(2, 160, 64)
+    saved = A._blocks
+    A._blocks = None   # any use of the blocked torch composition would now raise
+
+    def penalty(attn):
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = attn(qq, kk, vv)
+        gq, gk, gv = torch.autograd.grad((out * w).sum(), (qq, kk, vv), create_graph=True)
+        loss = gq.square().sum() + (gk * gv).sum()
+        return torch.autograd.grad(loss, (qq, kk, vv))
+
+    try:
+        ours = penalty(lambda a, b, c: fhog.attention(a, b, c, True))
+    finally:
+        A._blocks = saved
+    ref = penalty(lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(a, b, c, is_causal=True))
+    for a, b in zip(ours, ref):
+        assert normalised_max_error(a, b) < 1e-4
 
 
 @pytest.mark.parametrize("causal", [False, True])
