@@ -287,6 +287,7 @@ const Tuning& tuning() {
       if (!strcmp(tok, "b8")) r.b8 = atoi(val) != 0;
       else if (!strcmp(tok, "order")) r.order = !strcmp(val, "tile") ? 1 : !strcmp(val, "slice") ? 0 : -1;
       else if (!strcmp(tok, "split")) r.split = atoi(val) != 0;
+      else if (!strcmp(tok, "dd64")) r.dd64 = atoi(val) != 0;
     }
     return r;
   }();

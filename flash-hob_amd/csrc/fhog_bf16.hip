@@ -365,6 +365,150 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   }
 }
 
+// ---- pass 1 with 64 stationary rows per wave -----------------------------------------------------------------------
+// The dd sweep keeps only Q and ddQ resident, so a wave has the registers for TWO 32-query blocks (128 resident
+// registers at d = 128, 64 for the two S-shaped accumulators of each block): every K or ddK operand read from LDS then
+// feeds twice the MFMAs (16 reads per 48 instead of per 24), and a staged tile serves twice the rows.
+// One 32-key step of such a wave; A0 / A1: the query block takes part (a block whose queries see no key of the tile
+// is left out at compile time). P overwrites S in place.
+template <bool F16, int D, bool A0, bool A1>
+__device__ __forceinline__ void dd_block64(const char* stage, const int* aoff, const bf16x8_t (&Qb)[2][D / 16],
+                                           const bf16x8_t (&ddQb)[2][D / 16], float c_scale_log2, const float* l_log2,
+                                           const bool* masked, const int* lo, const int* hi, float* red) {
+  constexpr int KK = D / 16, TILE = TS * 2 * D, NSTEP = 2 * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
+  constexpr bool act[2] = {A0, A1};
+  f32x16_t sc[2] = {{0}, {0}}, dds[2] = {{0}, {0}};
+  bf16x8_t a[NB];
+#pragma unroll
+  for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + (i / KK) * TILE, aoff[i % KK]);
+#pragma unroll
+  for (int i = 0; i < NSTEP; i++) {
+    const int ph = i / KK, kk = i % KK, c = i % NB;
+    if (i + PF < NSTEP) a[(i + PF) % NB] = lds_read128(stage + ((i + PF) / KK) * TILE, aoff[(i + PF) % KK]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ph == 0) {   // A = K: S += K Q^T, ddS += K ddQ^T
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+        if (act[rb]) sc[rb] = mfma<F16>(a[c], Qb[rb][kk], sc[rb]);
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+        if (act[rb]) dds[rb] = mfma<F16>(a[c], ddQb[rb][kk], dds[rb]);
+    } else {         // A = ddK: ddS += ddK Q^T, and P = exp2(S c - L) behind the MFMAs
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+        if (act[rb]) dds[rb] = mfma<F16>(a[c], Qb[rb][kk], dds[rb]);
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+        if (act[rb]) {
+#pragma unroll
+          for (int r = EPK * kk; r < EPK * (kk + 1); r++) sc[rb][r] = __builtin_amdgcn_exp2f(sc[rb][r] * c_scale_log2 - l_log2[rb]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+    if (act[rb]) {
+      if (masked[rb]) {   // wave-uniform: the block holds hidden keys (mask edge or tensor end)
+        keep_branch();
+#pragma unroll
+        for (int r = 0; r < 16; r++) sc[rb][r] = in_limits(r, lo[rb], hi[rb]) ? sc[rb][r] : 0.f;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) red[rb] = __builtin_fmaf(sc[rb][r], dds[rb][r], red[rb]);   // scale applied once at the end
+    }
+}
+
+// Four waves of 64 queries each: 256 queries per workgroup, two workgroups per CU. (Two-wave workgroups of 128 queries,
+// four per CU, measured 20-40 % slower than these.)
+template <bool F16, int D, int MASK>
+__global__ void __launch_bounds__(256, 2) dd_sweep64_bf16(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int ROWS = 256, NT = 2, TILE = TS * 2 * D, STAGE = NT * TILE, KK = D / 16;
+  int bh, tile;
+  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int q0 = tile * ROWS, qw = q0 + 64 * wave;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[NT] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff};
+
+  // d_i = sum_c O_ic dO_ic for the sweeps behind this one (fhog/triton_bwdbwd.py:580), before the resident operands
+  // are loaded: its operands are dead by then
+  int qi[2];
+  int64_t row[2];
+  float l_log2[2];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) {
+    qi[rb] = qw + 32 * rb + n;
+    const int qr = min(qi[rb], p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
+    row[rb] = (int64_t)bh * p.n_q + qr;
+    bf16x8_t Ob[KK], dOb[KK];
+    load_resident<D>(Ob, (const __bf16*)p.o + qoff, p.stride_qn, qr, h);
+    load_resident<D>(dOb, (const __bf16*)p.dO + qoff, p.stride_qn, qr, h);
+    float dsum = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(to_f32<F16>(Ob[kk][e]), to_f32<F16>(dOb[kk][e]), dsum);
+    dsum += __shfl_xor(dsum, 32);
+    if (h == 0 && qi[rb] < p.n_q) p.ws_d[row[rb]] = dsum;
+    l_log2[rb] = p.lse[row[rb]] * kLog2e;
+  }
+  bf16x8_t Qb[2][KK], ddQb[2][KK];
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) {
+    const int qr = min(qi[rb], p.n_q - 1);
+    load_resident<D>(Qb[rb], (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
+    load_resident<D>(ddQb[rb], (const __bf16*)p.ddq + qoff, p.stride_qn, qr, h);
+  }
+  const float c_scale_log2 = p.scale * kLog2e;
+  wait_vm0();   // the staging loads below are invisible to the compiler's wait counts (see q_sweep_bf16)
+
+  int aoff[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;
+  geo.tile_range(q0, ROWS, j_begin, j_end);
+  Dma<D> dma;
+  dma.init(p.stride_kn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  const auto stage_tile = [&](int j) {
+    dma.template issue_all<NT>(ring_lds + (j & 1) * STAGE, TILE, src, (int64_t)j * TS * p.stride_kn, wave, p.n_k - j * TS);
+  };
+  if (j_begin < j_end) stage_tile(j_begin);
+  dma_wait();
+  __syncthreads();
+
+  float red[2] = {0.f, 0.f};
+  for (int j = j_begin; j < j_end; j++) {
+    if (j + 1 < j_end) stage_tile(j + 1);
+    const int k0 = j * TS;
+    bool act[2], masked[2];
+    int lo[2] = {0, 0}, hi[2] = {0, 0};   // key k0 + 8g + 4h + e is visible to the lane's query of block rb iff lo <= 8g + e <= hi
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+      act[rb] = !geo.dead(k0, qw + 32 * rb);
+      masked[rb] = act[rb] && geo.partial(k0, qw + 32 * rb);
+      if (masked[rb]) keep_branch(), geo.limits(k0, qi[rb], h, lo[rb], hi[rb]);
+    }
+    const char* stage = smem + (j & 1) * STAGE;
+    if (act[0] && act[1]) dd_block64<F16, D, true, true>(stage, aoff, Qb, ddQb, c_scale_log2, l_log2, masked, lo, hi, red);
+    else if (act[1]) dd_block64<F16, D, false, true>(stage, aoff, Qb, ddQb, c_scale_log2, l_log2, masked, lo, hi, red);
+    else if (MASK == MASK_BAND && act[0]) dd_block64<F16, D, true, false>(stage, aoff, Qb, ddQb, c_scale_log2, l_log2, masked, lo, hi, red);
+    dma_wait();
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) {
+    float r = red[rb];
+    r += __shfl_xor(r, 32);
+    if (h == 0 && qi[rb] < p.n_q) p.ws_dd[row[rb]] = r * p.scale;
+  }
+}
+
 // Pass 4 (dK2, dV2) at d = 64 as a single-role kernel: 256 threads = 4 waves own 128 keys (K, ddK, V, ddV rows in
 // registers), Q-side tiles of 32 queries stream through a two-stage LDS ring together with the four row statistics of
 // those queries. First-level products have the queries as M and the keys as N, so a lane owns one key and its
@@ -609,6 +753,15 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
       if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
       return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
     }
+  }
+  // Pass 1 at d = 128 with 64 queries per wave (256 per workgroup) once the launch has 2048 such workgroups (four rounds of
+  // two per CU): half the LDS operand reads per MFMA, 4.7 % faster on 32 x 16384 rows. Smaller masked launches lose more
+  // to the coarser balance than the reads gain (32 x 4096 rows: 512 workgroups, all resident at once, +9 %), and at
+  // d = 64 the 32-query kernel with its three waves per SIMD is faster.
+  if constexpr (D == 128) {
+    const int dd64 = tuning().dd64;
+    if (pass == FHOG_PASS_DD && !split && (dd64 < 0 ? g8 >= 2048 : dd64 == 1))
+      return launch_sweep(dd_sweep64_bf16<F16, D, MASK>, g8, 2 * 2 * tile, s, p, 256);
   }
   switch (pass) {
     case FHOG_PASS_DD:

@@ -58,8 +58,9 @@ struct Params {
 //                      (default: 8 waves when that still gives 512 workgroups)
 //   order=slice|tile   workgroup order within an XCD (default: tile-major with a mask, slice after slice without)
 //   split=0|1          let small launches split their streamed side (default 1)
+//   dd64=0|1           dd sweep at d = 128: 32 | 64 queries per wave (default: 64 when that still gives 2048 workgroups)
 struct Tuning {
-  int b8 = -1, order = -1, split = 1;
+  int b8 = -1, order = -1, split = 1, dd64 = -1;
 };
 const Tuning& tuning();
 

@@ -392,6 +392,30 @@ def test_many_slices_d128_statistics_in_256_row_workgroups(case, fused_stats):
         assert normalised_max_error(a, b) < 1e-2, name
 
 
+@pytest.mark.parametrize("case", [(520, 1000, 1000, "causal", None, torch.bfloat16), (512, 1021, 515, "none", None, torch.float16),
+                                  (700, 770, 1100, "bottom_right", 300, torch.bfloat16)])
+def test_many_rows_d128_dd_sweep_with_64_queries_per_wave(case):
+    """At d = 128 a dd sweep of at least 2048 workgroups of 256 query rows runs 64 queries per wave (two 32-query blocks,
+    either of which a mask can leave out of a step): ragged ends, masks and dtypes; d and dd against the fp64 closed form
+    on sampled slices and against the fp32-MFMA kernels on all of them, outputs against fp32 autograd on sampled slices."""
+    batch, n_q, n_k, kind, window, dtype = case
+    causal = {"none": False, "causal": True, "bottom_right": "bottom_right"}[kind]
+    x = make_case(batch, n_q, n_k, 128, dtype, seed=78, grad_std=0.1)
+    scale = 128 ** -0.5
+    x = with_caches(x, scale, causal, window)
+    fast = run_fhog(x, scale, causal, window=window, impl="bf16", return_stats=True)
+    slow = run_fhog(x, scale, causal, window=window, impl="fp32", return_stats=True)
+    heads = [0, batch // 2, batch - 1]
+    ref = reference_fp32_gpu(x, scale, causal, heads=heads, window=window)
+    ref64 = reference_fp64_cpu(x, scale, causal, window, heads=heads[-2:])
+    e = errors([o[heads] for o in fast[:4]], ref)
+    assert max(e.values()) < 2e-2, e
+    for got, name in zip(fast[4], ("d", "dd", "b")):
+        assert normalised_max_error(got[heads[-2:]], ref64[name]) < 1e-2, name
+    for a, b, name in zip(fast[4], slow[4], ("d", "dd", "b")):
+        assert normalised_max_error(a, b) < 1e-2, name
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("impl", ["bf16", "fp32"])
 @pytest.mark.parametrize("shape", [(2, 256, 128, 64), (3, 384, 384, 128)])
