@@ -78,6 +78,16 @@ extern "C" {
 #define FHOG_SCHEDULE_FUSED_STATS 1 /* opt-in: dd and b from one sweep (FHOG_PASS_DD_B), 22 recomputed products;
                                        b differs from the four-pass value only by fp32 summation order */
 
+/* Launch choices (the counterpart of the reference's autotune list, fhog/triton_bwdbwd.py:12-36) are fixed functions of
+ * the launch size. For experiments they can be overridden through the environment variable FHOG_TUNE, a comma-separated
+ * list of key=value read once, on the host, at the first launch of the process (never in a timed path):
+ *   b8=0|1            b and dd+b sweeps at d = 128: 128-row workgroups of 4 waves | 256-row workgroups of 8 waves
+ *   order=slice|tile  workgroup order within an XCD: one (batch*head) slice after the other | the slices of an XCD advance
+ *                     through their tiles together
+ *   split=0|1         small launches may split their streamed side over several workgroups (needs the workspace of
+ *                     fhog_bwdbwd_workspace_hint)
+ *   dd64=0|1          dd sweep at d = 128 with 32 | 64 queries per wave
+ * Results do not depend on any of them beyond fp32 summation order (split) - the others are bit-identical. */
 typedef struct fhog_bwdbwd_args {
   /* inputs (device pointers); q, o, dO, ddq: (batch, n_q, d); k, v, ddk, ddv: (batch, n_k, d) */
   const void* q;
