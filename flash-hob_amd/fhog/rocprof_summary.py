@@ -38,7 +38,7 @@ def pass_of(kernel):
     m = re.match(r"q_sweep_bf16<\w+, \d+, (\d)", kernel)
     if m:
         return int(m.group(1))
-    for prefix, p in (("q_sweep3_pc", 3), ("k_sweep_pc", 4), ("k_sweep_bf16", 4), ("rowdot", 0), ("attn_fwd", "fwd"),
+    for prefix, p in (("dd_sweep64_bf16", 1), ("q_sweep3_pc", 3), ("k_sweep_pc", 4), ("k_sweep_bf16", 4), ("rowdot", 0), ("attn_fwd", "fwd"),
                       ("attn_bwd_q", "bwd_q"), ("attn_bwd_k", "bwd_k")):
         if kernel.startswith(prefix):
             return p
