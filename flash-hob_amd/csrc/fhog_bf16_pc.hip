@@ -133,6 +133,128 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
 }
 
 
+// Consumer wave of pass 3: the second-level products of one output, OUT = 0: dQ2 = dS ddK + dS' K, OUT = 1:
+// ddO = ddP V + P ddV, for the 64 queries of the pair qp = wq / 2 and all D columns (eight 32 x 32 accumulators). Per
+// 32-key block it reads two of the four operand tiles of its two query blocks and two of the four staged tensors: each
+// transposed K-side operand feeds two MFMAs (one per query block), each S-shaped operand D / 32 of them (one per column
+// block), 24 KiB of LDS reads per block where a 64 x 64 block of BOTH outputs takes 32 KiB. The wave also issues the
+// staging loads of its quarter of every tile.
+template <bool F16, int D, int MASK, int OUT>
+__device__ __forceinline__ void consume_q(const Params& p, char* smem, const StreamKeys<MASK>& geo, int j_begin, int j_end,
+                                          int q0, int wq, int lane, int split, int bh) {
+  using SM = PCSmem<D, false>;
+  constexpr int NC = D / 32;
+  // operand tiles: dS, dS', ddP, P; staged tensors: K, ddK, V, ddV
+  constexpr int A0 = OUT ? 2 : 0, A1 = OUT ? 3 : 1, B0 = OUT ? 2 : 1, B1 = OUT ? 3 : 0;
+  const int n = lane & 31, h = lane >> 5, qp = wq >> 1;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
+                          (const __bf16*)p.ddv + koff};
+  f32x16_t acc[2][NC];  // [query block of the pair][32-column block]
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++) acc[qb][cb] = f32x16_t{0};
+  int troff[NC][2];
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  const int qw0 = q0 + 64 * qp;            // first query of the pair
+  const char* sop_pair = smem + SM::SOP_BASE + (2 * qp) * SM::SOP_WAVE;
+  Dma<D> dma;
+  dma.init(p.stride_kn, wq, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  if (j_begin < j_end)
+    dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
+  dma_wait();
+  __syncthreads();
+  int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
+  for (int j = j_begin; j <= j_end; j++) {
+    if (j + 1 < j_end) {
+      const uint32_t dst = ring_lds + sn * SM::STAGE;
+      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
+      dma.template issue_all<4>(dst, SM::TILE, src, adv, wq, p.n_k - (j + 1) * TS);
+    }
+    // block j-1: query block qb of the pair took part iff the tile held a key visible to it
+    const bool act0 = j > j_begin && !geo.dead((j - 1) * TS, qw0);
+    const bool act1 = j > j_begin && !geo.dead((j - 1) * TS, qw0 + 32);
+    const bool act = act0 || act1;
+    const char* stage = smem + sc * SM::STAGE;
+    const char* sop = sop_pair + ((j - 1) & 1) * SM::SOP_BUF;
+    // two column blocks per iteration (k-step t, column pair cp): the four MFMAs on one accumulator are four instructions apart
+    constexpr int NIT = 2 * (NC / 2);
+    bf16x8_t bop[2][2][2];   // [buffer][column block of the pair][product]
+    bf16x8_t a_op[2][2][2];  // [k-step][query block][product]
+    const auto read_b = [&](int buf, int it) {
+      const int t = it / (NC / 2), cp = it % (NC / 2);
+#pragma unroll
+      for (int cl = 0; cl < 2; cl++) {
+        const char* b0 = stage + troff[2 * cp + cl][0];
+        const char* b1 = stage + troff[2 * cp + cl][1];
+        bop[buf][cl][0] = lds_read_tr_pre(b0, b1, B0 * SM::TILE + t * 16 * 2 * D);
+        bop[buf][cl][1] = lds_read_tr_pre(b0, b1, B1 * SM::TILE + t * 16 * 2 * D);
+      }
+    };
+    if (act) {
+      read_b(0, 0);
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+          a_op[t][qb][0] = sop_read(sop + qb * SM::SOP_WAVE + A0 * SOP_TILE, t, lane);
+          a_op[t][qb][1] = sop_read(sop + qb * SM::SOP_WAVE + A1 * SOP_TILE, t, lane);
+        }
+#pragma unroll
+      for (int it = 0; it < NIT; it++) {
+        const int t = it / (NC / 2), cp = it % (NC / 2), c = it & 1;
+        if (it + 1 < NIT) read_b(c ^ 1, it + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pr = 0; pr < 2; pr++)
+#pragma unroll
+          for (int cl = 0; cl < 2; cl++) {
+            if (act0) acc[0][2 * cp + cl] = mfma<F16>(a_op[t][0][pr], bop[c][cl][pr], acc[0][2 * cp + cl]);
+            // with a plain causal mask (or none) a tile that block 0 takes part in is also one for block 1
+            if (MASK != MASK_BAND || act1) acc[1][2 * cp + cl] = mfma<F16>(a_op[t][1][pr], bop[c][cl][pr], acc[1][2 * cp + cl]);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    dma_wait();
+    __syncthreads();
+    sc = (sc == RING - 1) ? 0 : sc + 1;
+    sn = (sn == RING - 1) ? 0 : sn + 1;
+  }
+  // acc[qb][cb][r] holds (query qw0 + 32 qb + 8*(r/4) + 4h + r%4, column 32 cb + n)
+  if (p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]; combine_out finishes the pass
+    const int64_t rows = (int64_t)p.batch * p.n_q;
+    float* pq = p.part + ((int64_t)split * 2 * rows + (OUT ? rows : 0) + (int64_t)bh * p.n_q) * D;
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+      for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
+          if (qrow < p.n_q) pq[(int64_t)qrow * D + 32 * cb + n] = acc[qb][cb][r];
+        }
+    return;
+  }
+  uint16_t* o = (uint16_t*)(OUT ? p.ddo : p.dq2) + qoff;
+  const float f = OUT ? 1.f : p.scale;
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
+        if (qrow < p.n_q) o[(int64_t)qrow * p.stride_qn + 32 * cb + n] = to_elem<F16>(acc[qb][cb][r] * f);
+      }
+}
+
 template <bool F16, int D, int MASK>
 __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -182,138 +304,9 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
       sp = (sp == RING - 1) ? 0 : sp + 1;
     }
   } else {
-    // consumer wave cw owns the 64 x 64 output block (query pair qp, column half ch): every transposed
-    // K-side operand read from LDS feeds two MFMAs (one per 32-query block of the pair)
-    const int qp = wq >> 1, ch = wq & 1;
-    const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
-                            (const __bf16*)p.ddv + koff};
-    f32x16_t acc_dq[2][2], acc_ddo[2][2];  // [query block of the pair][32-column block of the half]
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-      for (int cl = 0; cl < 2; cl++) {
-        acc_dq[qb][cl] = f32x16_t{0};
-        acc_ddo[qb][cl] = f32x16_t{0};
-      }
-    int troff[2][2];
-#pragma unroll
-    for (int cl = 0; cl < 2; cl++) {
-      troff[cl][0] = tr_lane_off_acc<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 0, lane);
-      troff[cl][1] = tr_lane_off_acc<D>((D == 128 ? 2 * ch : ch) + (D == 128 ? cl : 0), 1, lane);
-    }
-    constexpr int NCL = (D == 128) ? 2 : 1;  // 32-column blocks per consumer wave
-    const int qw0 = q0 + 64 * qp;            // first query of the pair
-    const char* sop_pair = smem + SM::SOP_BASE + (2 * qp) * SM::SOP_WAVE;
-    Dma<D> dma;
-    dma.init(p.stride_kn, wq, lane);
-    const uint32_t ring_lds = lds_addr(smem);
-    if (j_begin < j_end)
-      dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
-    dma_wait();
-    __syncthreads();
-    int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
-    for (int j = j_begin; j <= j_end; j++) {
-      if (j + 1 < j_end) {
-        const uint32_t dst = ring_lds + sn * SM::STAGE;
-        const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-        dma.template issue_all<4>(dst, SM::TILE, src, adv, wq, p.n_k - (j + 1) * TS);
-      }
-      // block j-1: query block qb of the pair took part iff the tile held a key visible to it
-      const bool act0 = j > j_begin && !geo.dead((j - 1) * TS, qw0);
-      const bool act1 = j > j_begin && !geo.dead((j - 1) * TS, qw0 + 32);
-      if (act0 || act1) {
-        const char* stage = smem + sc * SM::STAGE;
-        const char* sop = sop_pair + ((j - 1) & 1) * SM::SOP_BUF;
-        const char* bp[NCL][2];
-#pragma unroll
-        for (int cl = 0; cl < NCL; cl++) {
-          bp[cl][0] = stage + troff[cl][0];
-          bp[cl][1] = stage + troff[cl][1];
-        }
-        // operand order in the stage: K, ddK, V, ddV; in the operand tiles: dS, dS', ddP, P
-        bf16x8_t bop[2][4];
-#pragma unroll
-        for (int x = 0; x < 4; x++) bop[0][x] = lds_read_tr_pre(bp[0][0], bp[0][1], x * SM::TILE);
-        bf16x8_t a_opt[2][2][4];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-          for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-            for (int x = 0; x < 4; x++) a_opt[t][qb][x] = sop_read(sop + qb * SM::SOP_WAVE + x * SOP_TILE, t, lane);
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-          const auto& a_op = a_opt[t];
-#pragma unroll
-          for (int cl = 0; cl < NCL; cl++) {
-            const int it = t * NCL + cl, c = it & 1;
-            if (it + 1 < 2 * NCL) {
-              const int t1 = (it + 1) / NCL, cl1 = (it + 1) % NCL;
-#pragma unroll
-              for (int x = 0; x < 4; x++)
-                bop[c ^ 1][x] = lds_read_tr_pre(bp[cl1][0], bp[cl1][1], x * SM::TILE + t1 * 16 * 2 * D);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (act0) {
-              acc_dq[0][cl] = mfma<F16>(a_op[0][0], bop[c][1], acc_dq[0][cl]);
-              acc_ddo[0][cl] = mfma<F16>(a_op[0][2], bop[c][2], acc_ddo[0][cl]);
-            }
-            // with a plain causal mask (or none) a tile that block 0 takes part in is also one for block 1
-            if (MASK != MASK_BAND || act1) {
-              acc_dq[1][cl] = mfma<F16>(a_op[1][0], bop[c][1], acc_dq[1][cl]);
-              acc_ddo[1][cl] = mfma<F16>(a_op[1][2], bop[c][2], acc_ddo[1][cl]);
-            }
-            if (act0) {
-              acc_dq[0][cl] = mfma<F16>(a_op[0][1], bop[c][0], acc_dq[0][cl]);
-              acc_ddo[0][cl] = mfma<F16>(a_op[0][3], bop[c][3], acc_ddo[0][cl]);
-            }
-            if (MASK != MASK_BAND || act1) {
-              acc_dq[1][cl] = mfma<F16>(a_op[1][1], bop[c][0], acc_dq[1][cl]);
-              acc_ddo[1][cl] = mfma<F16>(a_op[1][3], bop[c][3], acc_ddo[1][cl]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-      }
-      dma_wait();
-      __syncthreads();
-      sc = (sc == RING - 1) ? 0 : sc + 1;
-      sn = (sn == RING - 1) ? 0 : sn + 1;
-    }
-    // acc[qb][cl][r] holds (query qw0 + 32 qb + 8*(r/4) + 4h + r%4, column 32*(NCL*ch + cl) + n)
-    if (p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]; combine_out finishes the pass
-      const int64_t rows = (int64_t)p.batch * p.n_q;
-      float* pq = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_q) * D;
-#pragma unroll
-      for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-        for (int cl = 0; cl < NCL; cl++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
-            if (qrow < p.n_q) {
-              const int64_t o = (int64_t)qrow * D + 32 * (NCL * ch + cl) + n;
-              pq[o] = acc_dq[qb][cl][r];
-              pq[rows * D + o] = acc_ddo[qb][cl][r];
-            }
-          }
-      return;
-    }
-    uint16_t* odq = (uint16_t*)p.dq2 + qoff;
-    uint16_t* oddo = (uint16_t*)p.ddo + qoff;
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-      for (int cl = 0; cl < NCL; cl++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int qrow = qw0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
-          if (qrow < p.n_q) {
-            const int64_t o = (int64_t)qrow * p.stride_qn + 32 * (NCL * ch + cl) + n;
-            odq[o] = to_elem<F16>(acc_dq[qb][cl][r] * p.scale);
-            oddo[o] = to_elem<F16>(acc_ddo[qb][cl][r]);
-          }
-        }
+    // consumer wave (qp, out) owns the 64-query x D-column block of ONE output for the query pair qp
+    if (wq & 1) consume_q<F16, D, MASK, 1>(p, smem, geo, j_begin, j_end, q0, wq, lane, split, bh);
+    else consume_q<F16, D, MASK, 0>(p, smem, geo, j_begin, j_end, q0, wq, lane, split, bh);
   }
 }
 
