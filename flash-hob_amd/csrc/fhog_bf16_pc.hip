@@ -382,18 +382,28 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
     const __bf16* src[3] = {(const __bf16*)p.q + qoff, (const __bf16*)p.ddq + qoff, (const __bf16*)p.dO + qoff};
     const float* stat_src[4] = {p.lse + (int64_t)bh * p.n_q, p.ws_d + (int64_t)bh * p.n_q, p.ws_dd + (int64_t)bh * p.n_q,
                                 p.ws_b + (int64_t)bh * p.n_q};
-    f32x16_t acc_dk[NC], acc_dv[NC];
+    // consumer wave (kp, ch) owns the keys of the producer waves 2 kp and 2 kp + 1 and the column half ch of both outputs
+    // (eight 32 x 32 accumulators): every transposed Q-side operand read from LDS feeds the MFMAs of two key blocks, every
+    // S-shaped operand those of two column blocks - 24 KiB of LDS reads per block where one key block with all columns
+    // takes 30 KiB
+    constexpr int NCL = NC / 2;   // 32-column blocks per consumer wave
+    const int kp = wq >> 1, ch = wq & 1;
+    const int kw2 = k0 + 64 * kp;   // first key of the pair
+    f32x16_t acc_dk[2][NCL], acc_dv[2][NCL];   // [key block of the pair][column block of the half]
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++) {
-      acc_dk[cb] = f32x16_t{0};
-      acc_dv[cb] = f32x16_t{0};
-    }
-    int troff[NC][2];
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++) {
-      troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
-      troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+      for (int cl = 0; cl < NCL; cl++) {
+        acc_dk[kb][cl] = f32x16_t{0};
+        acc_dv[kb][cl] = f32x16_t{0};
+      }
+    int troff[NCL][2];
+#pragma unroll
+    for (int cl = 0; cl < NCL; cl++) {
+      troff[cl][0] = tr_lane_off_acc<D>(NCL * ch + cl, 0, lane);
+      troff[cl][1] = tr_lane_off_acc<D>(NCL * ch + cl, 1, lane);
     }
+    const char* sop_pair = smem + SM::SOP_BASE + (2 * kp) * SM::SOP_WAVE;
     const int sopoff[2] = {sop_tr_lane_off(0, lane), sop_tr_lane_off(1, lane)};
     Dma<D> dma;
     dma.init(p.stride_qn, wq, lane);
@@ -425,37 +435,51 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
         load_stat((j + 1) * TS);
         dma.template issue_all<3>(dst, SM::TILE, src, adv, wq, p.n_q - (j + 1) * TS);
       }
-      if (j > t_begin && !geo.dead((j - 1) * TS, kw)) {
+      // block j-1: key block kb of the pair took part iff the tile held a query that sees one of its keys
+      const bool act0 = j > t_begin && !geo.dead((j - 1) * TS, kw2);
+      const bool act1 = j > t_begin && !geo.dead((j - 1) * TS, kw2 + 32);
+      if (act0 || act1) {
         const char* stage = smem + sc * SM::STAGE;
-        const char* sop = sop_base + ((j - 1) & 1) * SM::SOP_BUF;
-        const char* bp[NC][2];
+        const char* sop = sop_pair + ((j - 1) & 1) * SM::SOP_BUF;
+        const char* bp[NCL][2];
 #pragma unroll
-        for (int cb = 0; cb < NC; cb++) {
-          bp[cb][0] = stage + troff[cb][0];
-          bp[cb][1] = stage + troff[cb][1];
+        for (int cl = 0; cl < NCL; cl++) {
+          bp[cl][0] = stage + troff[cl][0];
+          bp[cl][1] = stage + troff[cl][1];
         }
-        bf16x8_t a_op[2][3];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-          for (int x = 0; x < 3; x++) a_op[t][x] = lds_read_tr_pre(sop + sopoff[0], sop + sopoff[1], x * SOP_TILE + t * 16 * 64);
+        // operand tiles: dS, dS', ddP; staged tensors: Q, ddQ, dO.  dK2^T += ddQ^T dS + Q^T dS' ; dV2^T += dO^T ddP
         bf16x8_t bop[2][3];
         bop[0][0] = lds_read_tr_pre(bp[0][0], bp[0][1], 1 * SM::TILE + 0 * 16 * 2 * D);
         bop[0][1] = lds_read_tr_pre(bp[0][0], bp[0][1], 0 * SM::TILE + 0 * 16 * 2 * D);
         bop[0][2] = lds_read_tr_pre(bp[0][0], bp[0][1], 2 * SM::TILE + 0 * 16 * 2 * D);
+        bf16x8_t a_op[2][2][3];   // [key block][k-step][tile]
 #pragma unroll
-        for (int it = 0; it < 2 * NC; it++) {
-          const int t = it / NC, cb = it % NC, c = it & 1;
-          if (it + 1 < 2 * NC) {
-            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
-            bop[c ^ 1][0] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 1 * SM::TILE + t1 * 16 * 2 * D);
-            bop[c ^ 1][1] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 0 * SM::TILE + t1 * 16 * 2 * D);
-            bop[c ^ 1][2] = lds_read_tr_pre(bp[cb1][0], bp[cb1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+          for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int x = 0; x < 3; x++)
+              a_op[kb][t][x] = lds_read_tr_pre(sop + kb * SM::SOP_WAVE + sopoff[0], sop + kb * SM::SOP_WAVE + sopoff[1], x * SOP_TILE + t * 16 * 64);
+#pragma unroll
+        for (int it = 0; it < 2 * NCL; it++) {
+          const int t = it / NCL, cl = it % NCL, c = it & 1;
+          if (it + 1 < 2 * NCL) {
+            const int t1 = (it + 1) / NCL, cl1 = (it + 1) % NCL;
+            bop[c ^ 1][0] = lds_read_tr_pre(bp[cl1][0], bp[cl1][1], 1 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][1] = lds_read_tr_pre(bp[cl1][0], bp[cl1][1], 0 * SM::TILE + t1 * 16 * 2 * D);
+            bop[c ^ 1][2] = lds_read_tr_pre(bp[cl1][0], bp[cl1][1], 2 * SM::TILE + t1 * 16 * 2 * D);
           }
           __builtin_amdgcn_sched_barrier(0);
-          acc_dk[cb] = mfma<F16>(a_op[t][0], bop[c][0], acc_dk[cb]);
-          acc_dv[cb] = mfma<F16>(a_op[t][2], bop[c][2], acc_dv[cb]);
-          acc_dk[cb] = mfma<F16>(a_op[t][1], bop[c][1], acc_dk[cb]);
+          if (act0) {
+            acc_dk[0][cl] = mfma<F16>(a_op[0][t][0], bop[c][0], acc_dk[0][cl]);
+            acc_dv[0][cl] = mfma<F16>(a_op[0][t][2], bop[c][2], acc_dv[0][cl]);
+          }
+          if (act1) {
+            acc_dk[1][cl] = mfma<F16>(a_op[1][t][0], bop[c][0], acc_dk[1][cl]);
+            acc_dv[1][cl] = mfma<F16>(a_op[1][t][2], bop[c][2], acc_dv[1][cl]);
+          }
+          if (act0) acc_dk[0][cl] = mfma<F16>(a_op[0][t][1], bop[c][1], acc_dk[0][cl]);
+          if (act1) acc_dk[1][cl] = mfma<F16>(a_op[1][t][1], bop[c][1], acc_dk[1][cl]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -465,35 +489,40 @@ __global__ void __launch_bounds__(PC_THREADS) k_sweep_pc(Params p) {
       sc = (sc == RING - 1) ? 0 : sc + 1;
       sn = (sn == RING - 1) ? 0 : sn + 1;
     }
+    // acc[kb][cl][r] holds (key kw2 + 32 kb + 8*(r/4) + 4h + r%4, column 32 (NCL ch + cl) + n)
     if (p.n_split > 1) {   // fp32 partial rows [split][dK2 | dV2][batch * n_k][D]
       const int64_t rows = (int64_t)p.batch * p.n_k;
       float* pk = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_k) * D;
 #pragma unroll
-      for (int cb = 0; cb < NC; cb++)
+      for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int krow = kw + 8 * (r / 4) + 4 * h + (r % 4);
-          if (krow < p.n_k) {
-            const int64_t o = (int64_t)krow * D + cb * 32 + n;
-            pk[o] = acc_dk[cb][r];
-            pk[rows * D + o] = acc_dv[cb][r];
+        for (int cl = 0; cl < NCL; cl++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int krow = kw2 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+            if (krow < p.n_k) {
+              const int64_t o = (int64_t)krow * D + 32 * (NCL * ch + cl) + n;
+              pk[o] = acc_dk[kb][cl][r];
+              pk[rows * D + o] = acc_dv[kb][cl][r];
+            }
           }
-        }
       return;
     }
     uint16_t* odk = (uint16_t*)p.dk2 + koff;
     uint16_t* odv = (uint16_t*)p.dv2 + koff;
 #pragma unroll
-    for (int cb = 0; cb < NC; cb++)
+    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int krow = kw + 8 * (r / 4) + 4 * h + (r % 4);
-        if (krow < p.n_k) {
-          const int64_t o = (int64_t)krow * p.stride_kn + cb * 32 + n;
-          odk[o] = to_elem<F16>(acc_dk[cb][r] * p.scale);
-          odv[o] = to_elem<F16>(acc_dv[cb][r]);
+      for (int cl = 0; cl < NCL; cl++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int krow = kw2 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+          if (krow < p.n_k) {
+            const int64_t o = (int64_t)krow * p.stride_kn + 32 * (NCL * ch + cl) + n;
+            odk[o] = to_elem<F16>(acc_dk[kb][cl][r] * p.scale);
+            odv[o] = to_elem<F16>(acc_dv[kb][cl][r]);
+          }
         }
-      }
   }
 }
 
