@@ -4,12 +4,12 @@
 size) and the SQ counters behind the matrix-pipe occupancy.
 
     cd /tmp && export TMPDIR=/tmp && cd <repo>
-    W=cfg2_bf16_causal_4096_d128
-    rocprofv3 --kernel-trace --stats -d gpurun_out/prof_kt -o kt --output-format csv -- python3 bench.py --profile-only --workload $W --steps 20 --warmup 5
-    rocprofv3 --pmc FETCH_SIZE -d gpurun_out/prof_fetch -o f --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
-    rocprofv3 --pmc WRITE_SIZE -d gpurun_out/prof_write -o w --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
-    rocprofv3 --pmc SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_VALU_MFMA_COEXEC_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_LDS_IDX_ACTIVE SQ_LDS_BANK_CONFLICT -d gpurun_out/prof_sq -o s --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
-    python3 flash-hob_amd/fhog/rocprof_summary.py --workload $W --root gpurun_out > profiles/bwdbwd_kernels_$W.md
+    W=cfg2_bf16_causal_4096_d128; OUT=prof_out        # any scratch directory
+    rocprofv3 --kernel-trace --stats -d $OUT/prof_kt -o kt --output-format csv -- python3 bench.py --profile-only --workload $W --steps 20 --warmup 5
+    rocprofv3 --pmc FETCH_SIZE -d $OUT/prof_fetch -o f --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
+    rocprofv3 --pmc WRITE_SIZE -d $OUT/prof_write -o w --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
+    rocprofv3 --pmc SQ_BUSY_CYCLES SQ_WAVE_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_VALU_MFMA_COEXEC_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_LDS_IDX_ACTIVE SQ_LDS_BANK_CONFLICT -d $OUT/prof_sq -o s --output-format csv -- python3 bench.py --profile-only --workload $W --steps 3 --warmup 1
+    python3 flash-hob_amd/fhog/rocprof_summary.py --workload $W --root $OUT > profiles/bwdbwd_kernels_$W.md
 
 ``bench.py`` reads the HBM bytes of the dominant kernel back from the machine-readable comment this script writes.
 """
@@ -96,7 +96,7 @@ def main():
     from fhog.workloads import WORKLOADS
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", required=True)
-    ap.add_argument("--root", default="gpurun_out", help="directory holding prof_kt, prof_fetch, prof_write, prof_sq")
+    ap.add_argument("--root", default="prof_out", help="directory holding prof_kt, prof_fetch, prof_write, prof_sq")
     ap.add_argument("--note", default="", help="free text appended to the summary")
     ap.add_argument("--compare", nargs="+", metavar="LABEL@DIR", help="instead of a summary: one table over runs made under "
                     "different FHOG_TUNE settings (each DIR holds prof_kt, prof_fetch, prof_sq)")
