@@ -597,6 +597,23 @@ def test_headline_properties_linearity_zero_and_sdpa_case():
     torch.testing.assert_close(base[3][:, 0].float(), x["ddV"][:, 0].float(), rtol=1e-2, atol=1e-3)
 
 
+@pytest.mark.parametrize("name", ["cfg2_bf16_causal_4096_d128", "cfg4_bf16_cross_1024x8192_d64", "cfg3_bf16_causal_16384_d128"])
+def test_full_size_statistic_b_is_the_row_dot_of_dO_and_ddO(name):
+    """b_i = dO_i . ddO_i - d_i dd_i holds for the exact quantities, whatever the size: the row statistic the second sweep
+    leaves in the workspace against an output of the third sweep, at the full benchmark sizes (every slice, every row)."""
+    from fhog.workloads import WORKLOADS, make_inputs
+    w = WORKLOADS[name]
+    x = {n: t.flatten(0, 1) for n, t in make_inputs(w, 3, device="cuda:0").items()}
+    x = with_caches(x, w.scale, w.causal)
+    dq2, dk2, dv2, ddo, (d, dd, b) = run_fhog(x, w.scale, w.causal, return_stats=True)
+    rowdot = torch.zeros_like(b)
+    for h0 in range(0, ddo.shape[0], 8):   # in slices: the fp32 copies of a whole tensor are large at N = 16384
+        rowdot[h0:h0 + 8] = (x["dO"][h0:h0 + 8].float() * ddo[h0:h0 + 8].float()).sum(-1)
+    want = rowdot - d * dd
+    # ddO is rounded to bf16 (2^-9 relative) before the row dot: the bound scales with sum_c |dO ddO| of the row
+    assert normalised_max_error(b, want) < 1e-2, normalised_max_error(b, want)
+
+
 def test_peak_memory_is_linear_in_n():
     """Workspace + outputs only: 4 output tensors and 3 fp32 row vectors, nothing of size N_Q x N_K. The larger
     workspace for split launches adds partial results of fewer than 2 * 131072 * d floats, whatever N (the number of

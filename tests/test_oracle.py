@@ -86,6 +86,9 @@ def test_row_identities(causal):
     np.testing.assert_allclose(cf["d"], (p * dp).sum(-1), atol=1e-12)               # d = sum_j P dP
     b_alt = np.einsum("id,id->i", x["do"], p @ x["ddv"]) - 2 * cf["d"] * cf["dd"] + (p * dp * dds).sum(-1)
     np.testing.assert_allclose(cf["b"], b_alt, atol=1e-12)
+    # b_i = dO_i . ddO_i - d_i dd_i: the statistic of the second sweep is a row dot of an OUTPUT of the third
+    # (ddO = P ddV + P (ddS - dd) V and sum_j P_ij dP_ij = d_i), which ties the two passes together
+    np.testing.assert_allclose(cf["b"], np.einsum("id,id->i", x["do"], cf["ddo"]) - cf["d"] * cf["dd"], atol=1e-12)
     if causal:  # row 0 sees only key 0
         np.testing.assert_allclose(cf["dq2"][0], 0.0, atol=1e-13)
         np.testing.assert_allclose(cf["ddo"][0], x["ddv"][0], atol=1e-13)
