@@ -87,6 +87,28 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
                           (const __bf16*)p.ddv + koff};
 
+  // The first streamed tile is requested before the resident operands: the two round trips to memory overlap instead of
+  // following each other (a workgroup that visits four tiles spends most of its time in this prologue).
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;  // key tiles this workgroup visits
+  geo.tile_range(q0, ROWS, j_begin, j_end);
+  if (p.n_split > 1) split_range(split, p.n_split, j_begin, j_end);
+  // staging: four waves share the rows of a tile; with eight waves each group of four takes half of the tensors
+  constexpr int NLD = NW == 8 ? NT / 2 : NT;
+  const int half = NW == 8 ? wave >> 2 : 0;
+  const __bf16* srcl[NLD];
+#pragma unroll
+  for (int x = 0; x < NLD; x++) {   // wave-uniform, and the staging instruction wants it in scalar registers
+    const uint64_t a = (uint64_t)(NW == 8 ? (half ? src[NT / 2 + x < NT ? NT / 2 + x : 0] : src[x]) : src[x]);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    srcl[x] = (const __bf16*)(((uint64_t)hi << 32) | lo);
+  }
+  Dma<D> dma;
+  dma.init(p.stride_kn, wave & 3, lane);
+  const uint32_t ring_lds = lds_addr(smem) + half * NLD * TILE;
+  if (j_begin < j_end)
+    dma.template issue_all<NLD>(ring_lds + (j_begin & 1) * STAGE, TILE, srcl, (int64_t)j_begin * TS * p.stride_kn, wave & 3, p.n_k - j_begin * TS);
+
   bf16x8_t Qb[KK], ddQb[KK], dOb[KK];
   load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
   load_resident<D>(ddQb, (const __bf16*)p.ddq + qoff, p.stride_qn, qr, h);
@@ -138,25 +160,6 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
 
-  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
-  int j_begin, j_end;  // key tiles this workgroup visits
-  geo.tile_range(q0, ROWS, j_begin, j_end);
-  if (p.n_split > 1) split_range(split, p.n_split, j_begin, j_end);
-  // staging: four waves share the rows of a tile; with eight waves each group of four takes half of the tensors
-  constexpr int NLD = NW == 8 ? NT / 2 : NT;
-  const int half = NW == 8 ? wave >> 2 : 0;
-  const __bf16* srcl[NLD];
-#pragma unroll
-  for (int x = 0; x < NLD; x++) {   // wave-uniform, and the staging instruction wants it in scalar registers
-    const uint64_t a = (uint64_t)(NW == 8 ? (half ? src[NT / 2 + x < NT ? NT / 2 + x : 0] : src[x]) : src[x]);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
-    srcl[x] = (const __bf16*)(((uint64_t)hi << 32) | lo);
-  }
-  Dma<D> dma;
-  dma.init(p.stride_kn, wave & 3, lane);
-  const uint32_t ring_lds = lds_addr(smem) + half * NLD * TILE;
-  if (j_begin < j_end)
-    dma.template issue_all<NLD>(ring_lds + (j_begin & 1) * STAGE, TILE, srcl, (int64_t)j_begin * TS * p.stride_kn, wave & 3, p.n_k - j_begin * TS);
   dma_wait();
   __syncthreads();
 
@@ -434,6 +437,18 @@ __global__ void __launch_bounds__(256, 2) dd_sweep64_bf16(Params p) {
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[NT] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff};
 
+  // the first streamed tile is requested before anything else is loaded: the round trips to memory overlap
+  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
+  int j_begin, j_end;
+  geo.tile_range(q0, ROWS, j_begin, j_end);
+  Dma<D> dma;
+  dma.init(p.stride_kn, wave, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  const auto stage_tile = [&](int j) {
+    dma.template issue_all<NT>(ring_lds + (j & 1) * STAGE, TILE, src, (int64_t)j * TS * p.stride_kn, wave, p.n_k - j * TS);
+  };
+  if (j_begin < j_end) stage_tile(j_begin);
+
   // d_i = sum_c O_ic dO_ic for the sweeps behind this one (fhog/triton_bwdbwd.py:580), before the resident operands
   // are loaded: its operands are dead by then
   int qi[2];
@@ -469,16 +484,6 @@ __global__ void __launch_bounds__(256, 2) dd_sweep64_bf16(Params p) {
   int aoff[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) aoff[kk] = tile_off<D>(n, 2 * kk + h);
-  const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
-  int j_begin, j_end;
-  geo.tile_range(q0, ROWS, j_begin, j_end);
-  Dma<D> dma;
-  dma.init(p.stride_kn, wave, lane);
-  const uint32_t ring_lds = lds_addr(smem);
-  const auto stage_tile = [&](int j) {
-    dma.template issue_all<NT>(ring_lds + (j & 1) * STAGE, TILE, src, (int64_t)j * TS * p.stride_kn, wave, p.n_k - j * TS);
-  };
-  if (j_begin < j_end) stage_tile(j_begin);
   dma_wait();
   __syncthreads();
 
