@@ -59,13 +59,13 @@ int validate(const fhog_bwdbwd_args* a) {
   if (a->dtype != FHOG_DTYPE_BF16 && a->dtype != FHOG_DTYPE_FP32 && a->dtype != FHOG_DTYPE_FP16)
     return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
   if (a->impl != FHOG_IMPL_AUTO && a->impl != FHOG_IMPL_FP32 && a->impl != FHOG_IMPL_BF16)
-    return fail(FHOG_E_DTYPE, "unknown impl %d", a->impl);
+    return fail(FHOG_E_IMPL, "unknown impl %d", a->impl);
   if (a->schedule != FHOG_SCHEDULE_FOUR_PASS && a->schedule != FHOG_SCHEDULE_FUSED_STATS)
-    return fail(FHOG_E_DTYPE, "unknown schedule %d", a->schedule);
+    return fail(FHOG_E_SCHEDULE, "unknown schedule %d", a->schedule);
   if (a->batch < 1 || a->n_q < 1 || a->n_k < 1)
     return fail(FHOG_E_SHAPE, "batch, n_q, n_k must be >= 1 (got %lld, %lld, %lld)", (long long)a->batch, (long long)a->n_q,
                 (long long)a->n_k);
-  if (a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)a->batch);
+  if (a->batch > 65535) return fail(FHOG_E_SHAPE, "batch %lld above 65535 (batch * head slices) is not supported", (long long)a->batch);
   if (a->n_q > (1 << 24) || a->n_k > (1 << 24)) return fail(FHOG_E_SHAPE, "n_q/n_k above 2^24 not supported");
   if (a->batch * a->n_q >= (int64_t)1 << 31) return fail(FHOG_E_SHAPE, "batch*n_q must be below 2^31");
   if (a->d != 32 && a->d != 64 && a->d != 128) return fail(FHOG_E_SHAPE, "head dim %lld not in {32, 64, 128}", (long long)a->d);
@@ -277,17 +277,33 @@ const Tuning& tuning() {
     const char* env = getenv("FHOG_TUNE");
     if (!env) return r;
     char buf[256];
+    if (strlen(env) >= sizeof(buf)) fprintf(stderr, "libfhog_hip: FHOG_TUNE is longer than %zu characters; the rest is ignored\n", sizeof(buf) - 1);
     strncpy(buf, env, sizeof(buf) - 1);
     buf[sizeof(buf) - 1] = 0;
-    for (char* tok = strtok(buf, ","); tok; tok = strtok(nullptr, ",")) {
+    // 0 / 1 switches; anything else is reported and ignored
+    const auto flag = [](const char* key, const char* val, int* out) {
+      if (!strcmp(val, "0") || !strcmp(val, "1")) *out = val[0] - '0';
+      else fprintf(stderr, "libfhog_hip: FHOG_TUNE: value '%s' of '%s' is not 0 or 1; ignored\n", val, key);
+    };
+    char* save = nullptr;
+    for (char* tok = strtok_r(buf, ",", &save); tok; tok = strtok_r(nullptr, ",", &save)) {
       char* eq = strchr(tok, '=');
-      if (!eq) continue;
+      if (!eq) {
+        fprintf(stderr, "libfhog_hip: FHOG_TUNE: '%s' is not key=value; ignored\n", tok);
+        continue;
+      }
       *eq = 0;
       const char* val = eq + 1;
-      if (!strcmp(tok, "b8")) r.b8 = atoi(val) != 0;
-      else if (!strcmp(tok, "order")) r.order = !strcmp(val, "tile") ? 1 : !strcmp(val, "slice") ? 0 : -1;
-      else if (!strcmp(tok, "split")) r.split = atoi(val) != 0;
-      else if (!strcmp(tok, "dd64")) r.dd64 = atoi(val) != 0;
+      if (!strcmp(tok, "b8")) flag(tok, val, &r.b8);
+      else if (!strcmp(tok, "split")) flag(tok, val, &r.split);
+      else if (!strcmp(tok, "dd64")) flag(tok, val, &r.dd64);
+      else if (!strcmp(tok, "order")) {
+        if (!strcmp(val, "tile")) r.order = 1;
+        else if (!strcmp(val, "slice")) r.order = 0;
+        else fprintf(stderr, "libfhog_hip: FHOG_TUNE: order is 'slice' or 'tile', not '%s'; ignored\n", val);
+      } else {
+        fprintf(stderr, "libfhog_hip: FHOG_TUNE: unknown key '%s'; ignored\n", tok);
+      }
     }
     return r;
   }();
@@ -403,6 +419,8 @@ int fhog_bwdbwd_static_ws(const fhog_bwdbwd_args* args, void* hip_stream) {
   a.ws_bytes = FHOG_STATIC_WS_BYTES;   // small launches split their streamed side as far as the rest of the array allows
   return fhog_bwdbwd(&a, hip_stream);
 }
+
+size_t fhog_static_ws_bytes(void) { return (size_t)FHOG_STATIC_WS_BYTES; }
 
 int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream) {
   if (!out || !flops) return fail(FHOG_E_NULL, "out or flops is NULL");

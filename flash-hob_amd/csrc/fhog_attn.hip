@@ -393,11 +393,11 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
     }
 }
 
-template <typename K>
-hipError_t launch(K kernel, unsigned grid, int smem, hipStream_t s, const AttnParams& p) {
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+template <auto Kernel>
+hipError_t launch(unsigned grid, int smem, hipStream_t s, const AttnParams& p) {
+  const hipError_t e = allow_dynamic_lds<Kernel>(smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), smem, s, p);
+  hipLaunchKernelGGL(Kernel, dim3(grid), dim3(256), smem, s, p);
   return hipGetLastError();
 }
 
@@ -405,11 +405,11 @@ template <bool F16, int D, int MASK>
 hipError_t launch_attn_d(const AttnParams& p, int which, hipStream_t s) {
   constexpr int TILE = TS * 2 * D;
   switch (which) {
-    case 0: return launch(attn_fwd_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
-    case 1: return launch(attn_bwd_q_bf16<F16, D, MASK>, grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    case 0: return launch<attn_fwd_bf16<F16, D, MASK>>(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
+    case 1: return launch<attn_bwd_q_bf16<F16, D, MASK>>(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * 2 * TILE, s, p);
     default:
       if constexpr (D == 64)
-        return launch(attn_bwd_k_bf16<F16, D, MASK>, grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
+        return launch<attn_bwd_k_bf16<F16, D, MASK>>(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch), 2 * (2 * TILE + 2 * TS * 4), s, p);
       else
         return hipErrorInvalidValue;   // d = 128 is dispatched to the producer/consumer kernel before this point
   }

@@ -170,7 +170,7 @@ hipError_t launch_mode(const AttnParams& p, hipStream_t s) {
   const int smem = (int)((2 * Tile<D>::FLOATS + (KSIDE ? 2 * TR : 0)) * sizeof(float));
   const int n_tiles = (int)((n_rows + TR * 4 - 1) / (TR * 4));
   const dim3 grid(bf16k::grid_blocks(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch)), block(256);
-  const hipError_t e = hipFuncSetAttribute((const void*)attn_fp32<T, D, MODE, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  const hipError_t e = allow_dynamic_lds<attn_fp32<T, D, MODE, MASKED>>(smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL((attn_fp32<T, D, MODE, MASKED>), grid, block, smem, s, p);
   return hipGetLastError();

@@ -732,11 +732,11 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
     }
 }
 
-template <typename K>
-hipError_t launch_sweep(K kernel, unsigned grid, int smem, hipStream_t s, const Params& p, unsigned threads = 256) {
-  const hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+template <auto Kernel>
+hipError_t launch_sweep(unsigned grid, int smem, hipStream_t s, const Params& p, unsigned threads = 256) {
+  const hipError_t e = allow_dynamic_lds<Kernel>(smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem, s, p);
+  hipLaunchKernelGGL(Kernel, dim3(grid), dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
@@ -755,8 +755,8 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   if constexpr (D == 128) {
     const int b8 = tuning().b8;
     if (!split && (b8 < 0 ? g8 >= 512 : b8 == 1) && (pass == FHOG_PASS_B || pass == FHOG_PASS_DD_B)) {
-      if (pass == FHOG_PASS_B) return launch_sweep(q_sweep_bf16<F16, D, 2, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
-      return launch_sweep(q_sweep_bf16<F16, D, 5, MASK, 8>, g8, 2 * 4 * tile, s, p, 512);
+      if (pass == FHOG_PASS_B) return launch_sweep<q_sweep_bf16<F16, D, 2, MASK, 8>>(g8, 2 * 4 * tile, s, p, 512);
+      return launch_sweep<q_sweep_bf16<F16, D, 5, MASK, 8>>(g8, 2 * 4 * tile, s, p, 512);
     }
   }
   // Pass 1 at d = 128 with 64 queries per wave (256 per workgroup) once the launch has 2048 such workgroups (four rounds of
@@ -766,24 +766,24 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
   if constexpr (D == 128) {
     const int dd64 = tuning().dd64;
     if (pass == FHOG_PASS_DD && !split && (dd64 < 0 ? g8 >= 2048 : dd64 == 1))
-      return launch_sweep(dd_sweep64_bf16<F16, D, MASK>, g8, 2 * 2 * tile, s, p, 256);
+      return launch_sweep<dd_sweep64_bf16<F16, D, MASK>>(g8, 2 * 2 * tile, s, p, 256);
   }
   switch (pass) {
     case FHOG_PASS_DD:
-      e = launch_sweep(q_sweep_bf16<F16, D, 1, MASK>, gq, 2 * 2 * tile, s, p);
+      e = launch_sweep<q_sweep_bf16<F16, D, 1, MASK>>(gq, 2 * 2 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<1>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_B:
-      e = launch_sweep(q_sweep_bf16<F16, D, 2, MASK>, gq, 2 * 4 * tile, s, p);
+      e = launch_sweep<q_sweep_bf16<F16, D, 2, MASK>>(gq, 2 * 4 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<2>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_DD_B:
-      e = launch_sweep(q_sweep_bf16<F16, D, 5, MASK>, gq, 2 * 4 * tile, s, p);
+      e = launch_sweep<q_sweep_bf16<F16, D, 5, MASK>>(gq, 2 * 4 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<5>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_DQ_DDO:
       if constexpr (D == 64) {
-        e = launch_sweep(q_sweep_bf16<F16, D, 3, MASK>, gq, 2 * 4 * tile, s, p);
+        e = launch_sweep<q_sweep_bf16<F16, D, 3, MASK>>(gq, 2 * 4 * tile, s, p);
         if (e == hipSuccess && split)
           hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_q * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
                              p.batch, p.n_q, p.stride_qb, p.stride_qn, (uint16_t*)p.dq2, (uint16_t*)p.ddo, p.scale);
@@ -793,7 +793,7 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
       break;
     case FHOG_PASS_DK_DV:
       if constexpr (D == 64) {
-        e = launch_sweep(k_sweep_bf16<F16, D, MASK>, gk, 2 * (3 * tile + 4 * TS * 4), s, p);
+        e = launch_sweep<k_sweep_bf16<F16, D, MASK>>(gk, 2 * (3 * tile + 4 * TS * 4), s, p);
         if (e == hipSuccess && split)
           hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_k * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
                              p.batch, p.n_k, p.stride_kb, p.stride_kn, (uint16_t*)p.dk2, (uint16_t*)p.dv2, p.scale);

@@ -737,7 +737,7 @@ __global__ void __launch_bounds__(PC_THREADS) attn_bwd_k_pc(AttnParams p) {
 template <bool F16, int D, int MASK>
 hipError_t launch_attn_bwd_k_pc_d(const AttnParams& p, hipStream_t s) {
   const int smem = PCSmemAttn<D>::TOTAL;
-  const hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_k_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  const hipError_t e = allow_dynamic_lds<attn_bwd_k_pc<F16, D, MASK>>(smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL((attn_bwd_k_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch)), dim3(PC_THREADS), smem, s, p);
   return hipGetLastError();
@@ -749,12 +749,12 @@ hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
   hipError_t e;
   if (pass == FHOG_PASS_DQ_DDO) {
     const int smem = PCSmem<D, false>::TOTAL;
-    e = hipFuncSetAttribute((const void*)q_sweep3_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = allow_dynamic_lds<q_sweep3_pc<F16, D, MASK>>(smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((q_sweep3_pc<F16, D, MASK>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split)), block, smem, s, p);
   } else {
     const int smem = PCSmem<D, true>::TOTAL;
-    e = hipFuncSetAttribute((const void*)k_sweep_pc<F16, D, MASK>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = allow_dynamic_lds<k_sweep_pc<F16, D, MASK>>(smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_sweep_pc<F16, D, MASK>), dim3(grid_blocks((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch * p.n_split)), block, smem, s, p);
   }

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "fhog_hip.h"
 
 namespace fhog {
@@ -84,6 +86,23 @@ struct AttnParams {
   int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
   int32_t window;
 };
+
+// A kernel that uses more than 64 KiB of dynamic LDS needs its limit raised before the first launch. Done once per
+// kernel and device (not per launch: the call takes a lock in the runtime and must not run under stream capture, so
+// the first launch of a kernel on a device has to happen outside a capture).
+template <auto Kernel>
+inline hipError_t allow_dynamic_lds(int bytes) {
+  constexpr int kDevices = 64;
+  static std::atomic<int> granted[kDevices];   // zero-initialised: nothing granted yet
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool memo = dev >= 0 && dev < kDevices;
+  if (memo && granted[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+  e = hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && memo) granted[dev].store(bytes, std::memory_order_release);
+  return e;
+}
 
 // Launchers implemented in the kernel translation units. Each returns hipGetLastError().
 hipError_t launch_rowdot(const Params& p, int dtype, hipStream_t s);                 // pass 0

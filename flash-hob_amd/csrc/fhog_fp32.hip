@@ -335,7 +335,7 @@ hipError_t launch_sweep_ws(const Params& p, hipStream_t s) {
   const int smem = (int)(floats * sizeof(float));
   const int n_tiles = (int)((n_rows + TR * nw - 1) / (TR * nw));
   const dim3 grid(bf16k::grid_blocks(MASKED ? (n_tiles + 1) / 2 : n_tiles, p.batch)), block(256);
-  const hipError_t e = hipFuncSetAttribute((const void*)sweep_fp32<T, D, PASS, MASKED, WS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  const hipError_t e = allow_dynamic_lds<sweep_fp32<T, D, PASS, MASKED, WS>>(smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL((sweep_fp32<T, D, PASS, MASKED, WS>), grid, block, smem, s, p);
   return hipGetLastError();

@@ -17,11 +17,12 @@ IMPL_AUTO, IMPL_FP32, IMPL_BF16 = 0, 1, 2
 MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT = 0, 1, 2
 PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B = 0, 1, 2, 3, 4, 5
 ABI_VERSION = 4
-STATIC_WS_BYTES = 16 << 20
+STATIC_WS_BYTES = 16 << 20   # of a default build; `lib().fhog_static_ws_bytes()` tells what the loaded library holds
 
 ERROR_NAMES = {
     -1: "FHOG_E_NULL", -2: "FHOG_E_SHAPE", -3: "FHOG_E_DTYPE", -4: "FHOG_E_STRIDE", -5: "FHOG_E_ALIGN",
-    -6: "FHOG_E_CAUSAL", -7: "FHOG_E_PASS", -8: "FHOG_E_LAUNCH", -9: "FHOG_E_SCALE",
+    -6: "FHOG_E_CAUSAL", -7: "FHOG_E_PASS", -8: "FHOG_E_LAUNCH", -9: "FHOG_E_SCALE", -10: "FHOG_E_IMPL",
+    -11: "FHOG_E_SCHEDULE",
 }
 
 
@@ -82,6 +83,8 @@ def lib() -> ctypes.CDLL:
     L.fhog_bwdbwd.argtypes = [POINTER(BwdBwdArgs), c_void_p]
     L.fhog_bwdbwd_static_ws.restype = c_int
     L.fhog_bwdbwd_static_ws.argtypes = [POINTER(BwdBwdArgs), c_void_p]
+    L.fhog_static_ws_bytes.restype = c_size_t
+    L.fhog_static_ws_bytes.argtypes = []
     L.fhog_bwdbwd_pass.restype = c_int
     L.fhog_bwdbwd_pass.argtypes = [POINTER(BwdBwdArgs), c_int, c_void_p]
     L.fhog_last_error.restype = c_char_p

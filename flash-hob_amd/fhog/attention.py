@@ -20,6 +20,7 @@ The double-backward is always the HIP library.
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Optional, Tuple
 
 import ctypes
@@ -58,10 +59,16 @@ def _scores(q, k, scale, causal, r0, n_q=None, window=None):
 
 
 
-def _hip_args(q, k, v, scale, causal, window=None) -> Optional[_lib.AttnArgs]:
-    """Arguments for the HIP first-order kernels, or None when they do not cover these tensors."""
-    if not (q.is_cuda and q.dtype in _HIP_DTYPES and k.dtype == v.dtype == q.dtype):
-        return None
+class _NotCovered(Exception):
+    """The HIP first-order kernels do not take these arguments; the message says why."""
+
+
+def _hip_args(q, k, v, scale, causal, window=None) -> _lib.AttnArgs:
+    """Arguments for the HIP first-order kernels; raises _NotCovered when they do not cover these tensors."""
+    if not q.is_cuda:
+        raise _NotCovered("the tensors are not on a ROCm device")
+    if q.dtype not in _HIP_DTYPES or not (k.dtype == v.dtype == q.dtype):
+        raise _NotCovered(f"dtypes {q.dtype}, {k.dtype}, {v.dtype}: need one of bf16, fp16, fp32 for all tensors")
     a = _lib.AttnArgs()
     a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     a.batch, a.n_q, a.d = q.shape
@@ -78,20 +85,18 @@ def _same_layout(ts) -> bool:
 
 
 def _attention_forward_hip(q, k, v, scale, causal, window=None):
-    """O and L from ``fhog_attn_fwd``; None when the kernels do not cover the arguments."""
+    """O and L from ``fhog_attn_fwd``; raises _NotCovered when the kernels do not cover the arguments."""
     q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
     if not _same_layout([k, v]):
         k, v = k.contiguous(), v.contiguous()
     a = _hip_args(q, k, v, scale, causal, window)
-    if a is None:
-        return None
     L_ = _lib.lib()
     with torch.cuda.device(q.device):
         o = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
         lse = torch.empty(q.shape[0], q.shape[1], dtype=torch.float32, device=q.device)
         a.o, a.lse = o.data_ptr(), lse.data_ptr()
         if L_.fhog_attn_validate(ctypes.byref(a), 0) != 0:
-            return None
+            raise _NotCovered(L_.fhog_last_error().decode())
         _lib.check(L_.fhog_attn_fwd(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
     return o, lse
 
@@ -105,8 +110,8 @@ def _attention_backward_hip(q, k, v, o, do, L, scale, causal, window=None):
         ts_k = [t.contiguous() for t in ts_k]
     (q, o, do), (k, v) = ts_q, ts_k
     a = _hip_args(q, k, v, scale, causal, window)
-    if a is None or o.dtype != q.dtype or do.dtype != q.dtype:
-        return None
+    if o.dtype != q.dtype or do.dtype != q.dtype:
+        raise _NotCovered(f"O and dO have dtypes {o.dtype}, {do.dtype}: need {q.dtype} like Q")
     L_ = _lib.lib()
     with torch.cuda.device(q.device):
         lse = L.reshape(q.shape[0], q.shape[1]).to(torch.float32).contiguous()
@@ -117,9 +122,23 @@ def _attention_backward_hip(q, k, v, o, do, L, scale, causal, window=None):
         a.o, a.lse, a.dO = o.data_ptr(), lse.data_ptr(), do.data_ptr()
         a.dq, a.dk, a.dv, a.ws = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr()
         if L_.fhog_attn_validate(ctypes.byref(a), 1) != 0:
-            return None
+            raise _NotCovered(L_.fhog_last_error().decode())
         _lib.check(L_.fhog_attn_bwd(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
     return dq, dk, dv
+
+
+class TorchCompositionWarning(RuntimeWarning):
+    """A first-order call left the HIP kernels for the blocked torch composition (10-100x slower)."""
+
+
+def _second_path(func: str, entry: str, why: Exception, use_hip: Optional[bool]) -> None:
+    """The HIP kernel refused the arguments: an error under ``use_hip=True``, else a warning that names the reason
+    before the caller goes on to the blocked torch composition (never silently: the composition is 10-100x slower)."""
+    if use_hip:
+        raise ValueError(f"{entry} does not cover these arguments: {why}")
+    warnings.warn(f"fhog.{func}: {entry} does not cover these arguments ({why}); running the blocked torch composition "
+                  "instead, which is far slower. Pass use_hip=False to choose it on purpose.",
+                  TorchCompositionWarning, stacklevel=3)
 
 
 def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, window: Optional[int] = None,
@@ -130,8 +149,9 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, w
     and of ``produce_L`` (``fhog/triton_flash.py:252-258``), with causal support and without an
     (batch, N_Q, N_K) allocation.
 
-    ``use_hip``: None = the HIP kernel when it covers the arguments, else the blocked torch composition;
-    True = the HIP kernel or an error; False = the torch composition.
+    ``use_hip``: None = the HIP kernel; when it refuses the arguments (a non-positive scale with 16-bit tensors, strides
+    that are not multiples of 16 bytes, CPU tensors), a ``TorchCompositionWarning`` names the reason and the blocked
+    torch composition runs instead. True = the HIP kernel or a ``ValueError``; False = the torch composition.
     """
     if q.dim() == 4:
         B, H = q.shape[:2]
@@ -143,12 +163,10 @@ def attention_forward(q, k, v, scale: Optional[float] = None, causal=False, *, w
     mask_code(causal, window, n_q, n_k)  # raises on an inapplicable mask
     scale = d ** -0.5 if scale is None else scale
     if use_hip is not False:
-        res = _attention_forward_hip(q, k, v, scale, causal, window)
-        if res is not None:
-            return res
-        if use_hip:
-            raise ValueError("fhog_attn_fwd does not cover these tensors (bf16, fp16 or fp32 on the GPU, d in {32, 64, 128}, "
-                             "a positive scale for 16-bit tensors)")
+        try:
+            return _attention_forward_hip(q, k, v, scale, causal, window)
+        except _NotCovered as why:
+            _second_path("attention_forward", "fhog_attn_fwd", why, use_hip)
     o = torch.empty_like(q)
     L = torch.empty(batch, n_q, dtype=torch.float32, device=q.device)
     for hs, rs in _blocks(batch, n_q, n_k):
@@ -173,12 +191,10 @@ def attention_backward(q, k, v, o, do, L, scale: float, causal, *, window: Optio
     batch, n_q, d = q.shape
     n_k = k.shape[1]
     if use_hip is not False:
-        res = _attention_backward_hip(q, k, v, o, do, L, scale, causal, window)
-        if res is not None:
-            return res
-        if use_hip:
-            raise ValueError("fhog_attn_bwd does not cover these tensors (bf16, fp16 or fp32 on the GPU, d in {32, 64, 128}, "
-                             "a positive scale for 16-bit tensors)")
+        try:
+            return _attention_backward_hip(q, k, v, o, do, L, scale, causal, window)
+        except _NotCovered as why:
+            _second_path("attention_backward", "fhog_attn_bwd", why, use_hip)
     dq = torch.empty_like(q)
     dk = torch.zeros(k.shape, dtype=torch.float32, device=k.device)
     dv = torch.zeros(v.shape, dtype=torch.float32, device=v.device)

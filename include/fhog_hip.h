@@ -47,6 +47,8 @@ extern "C" {
 #define FHOG_E_PASS (-7)      /* unknown pass id */
 #define FHOG_E_LAUNCH (-8)    /* HIP reported an error at launch */
 #define FHOG_E_SCALE (-9)     /* scale is not finite (fhog_attn_fwd / fhog_attn_bwd: not finite or not positive) */
+#define FHOG_E_IMPL (-10)     /* unknown kernel family (fhog_bwdbwd_args.impl) */
+#define FHOG_E_SCHEDULE (-11) /* unknown pass schedule (fhog_bwdbwd_args.schedule) */
 
 /* pass ids for fhog_bwdbwd_pass */
 #define FHOG_PASS_D 0      /* d_i  = sum_c O_ic dO_ic                         (fhog/triton_bwdbwd.py:580)     */
@@ -87,7 +89,8 @@ extern "C" {
  *   split=0|1         small launches may split their streamed side over several workgroups (needs the workspace of
  *                     fhog_bwdbwd_workspace_hint)
  *   dd64=0|1          dd sweep at d = 128 with 32 | 64 queries per wave
- * Results do not depend on any of them beyond fp32 summation order (split) - the others are bit-identical. */
+ * Results do not depend on any of them beyond fp32 summation order (split) - the others are bit-identical. Unknown keys
+ * and values are reported on stderr and ignored. */
 typedef struct fhog_bwdbwd_args {
   /* inputs (device pointers); q, o, dO, ddq: (batch, n_q, d); k, v, ddk, ddv: (batch, n_k, d) */
   const void* q;
@@ -161,9 +164,16 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream);
    has room. Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (two streams, two
    threads) race on it; calls ordered on one stream do not. Nothing in the array has to start at zero: every word a
    pass reads was written earlier in the same call. The first call on a device looks the array's address up
-   (hipGetSymbolAddress); no call allocates, frees or synchronises. */
+   (hipGetSymbolAddress) and raises the dynamic-LDS limit of the kernels it launches (hipFuncSetAttribute): make one call
+   per device and tensor configuration OUTSIDE a stream capture before capturing the entry point into a HIP graph.
+   No call allocates, frees or synchronises. */
+#ifndef FHOG_STATIC_WS_BYTES   /* a build of the library may size the array differently (hipcc -DFHOG_STATIC_WS_BYTES=...) */
 #define FHOG_STATIC_WS_BYTES (16 << 20)
+#endif
 int fhog_bwdbwd_static_ws(const fhog_bwdbwd_args* args, void* hip_stream);
+
+/* Size in bytes of that array in the loaded library (FHOG_STATIC_WS_BYTES of its build). Host-only. */
+size_t fhog_static_ws_bytes(void);
 
 /* One pass only (FHOG_PASS_*), for per-pass tests and profiling. Passes read the
    workspace rows written by earlier passes (stage 2 of the reference reads dD, B, D the

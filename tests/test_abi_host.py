@@ -128,8 +128,8 @@ def test_validate_accepts_good(L):
     (lambda a: setattr(a, "n_k", 0), -2, "n_k"),
     (lambda a: setattr(a, "batch", 70000), -2, "batch"),
     (lambda a: setattr(a, "dtype", 7), -3, "dtype"),
-    (lambda a: setattr(a, "impl", 9), -3, "impl"),
-    (lambda a: setattr(a, "schedule", 2), -3, "schedule"),
+    (lambda a: setattr(a, "impl", 9), -10, "impl"),
+    (lambda a: setattr(a, "schedule", 9), -11, "schedule"),
     (lambda a: setattr(a, "stride_qn", 32), -4, "stride"),
     (lambda a: setattr(a, "stride_kn", 68), -4, "multiples"),
     (lambda a: (setattr(a, "stride_kn", (1 << 24) + 8), setattr(a, "stride_kb", 1 << 40)), -4, "2^24"),

@@ -158,7 +158,7 @@ def test_fp32_mfma_first_order_kernels(case, causal):
 
 def test_fp32_kernels_take_a_negative_scale_and_16_bit_ones_fall_back():
     """The fp32-MFMA forward scales the scores before it takes their maximum: any sign of the scale. The 16-bit forward
-    needs a positive one: use_hip=True raises, the default takes the torch composition."""
+    needs a positive one: use_hip=True raises, the default warns and takes the torch composition."""
     import fhog
     y = make_case(2, 128, 160, 64, torch.float32, seed=24)
     o, L = fhog.attention_forward(y["Q"], y["K"], y["V"], -0.2, False, use_hip=True)
@@ -166,9 +166,11 @@ def test_fp32_kernels_take_a_negative_scale_and_16_bit_ones_fall_back():
     assert normalised_max_error(o, o_ref) < 1e-4
     assert (L.double().cpu() - torch.from_numpy(l_ref)).abs().max() < 1e-4
     x = make_case(2, 128, 160, 64, torch.bfloat16, seed=24)
-    with pytest.raises(ValueError):
+    with pytest.raises(ValueError, match="positive scale"):
         fhog.attention_forward(x["Q"], x["K"], x["V"], -0.2, False, use_hip=True)
-    o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], -0.2, False)
+    from fhog.attention import TorchCompositionWarning
+    with pytest.warns(TorchCompositionWarning, match="positive scale"):   # never silently: the warning carries the library's reason
+        o, L = fhog.attention_forward(x["Q"], x["K"], x["V"], -0.2, False)
     o_ref, l_ref = forward_o_lse(_np(x["Q"]), _np(x["K"]), _np(x["V"]), -0.2, False)
     assert normalised_max_error(o, o_ref) < 1e-2
 

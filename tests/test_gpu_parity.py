@@ -550,8 +550,11 @@ def test_cfg2_bf16_causal_4096_d128_headline(seed):
     assert max(e.values()) < 2e-2, e
 
 
-def test_cfg2_headline_fused_statistics_schedule():
-    w, e = _full_config("cfg2_bf16_causal_4096_d128", 2, fused_stats=True)
+@pytest.mark.parametrize("name,heads", [("cfg1_bf16_nc_2048_d64", None), ("cfg2_bf16_causal_4096_d128", None),
+                                        ("cfg3_bf16_causal_16384_d128", [3, 30]), ("cfg4_bf16_cross_1024x8192_d64", None)])
+def test_full_size_configs_fused_statistics_schedule(name, heads):
+    """The opt-in schedule (dd and b from one sweep) on every 16-bit benchmark configuration at full size."""
+    w, e = _full_config(name, 2, heads=heads, fused_stats=True)
     assert max(e.values()) < 2e-2, e
 
 

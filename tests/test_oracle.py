@@ -92,6 +92,14 @@ def test_row_identities(causal):
     if causal:  # row 0 sees only key 0
         np.testing.assert_allclose(cf["dq2"][0], 0.0, atol=1e-13)
         np.testing.assert_allclose(cf["ddo"][0], x["ddv"][0], atol=1e-13)
+    # The key-side outputs sum to zero over the keys: dK2 = dS^T ddQ + dS'^T Q and dV2 = ddP^T dO, and every row of dS,
+    # dS' and ddP sums to zero over j. A probability that underflows on the device breaks exactly this (the long-N GPU
+    # test bounds the column sums of the device outputs with it).
+    np.testing.assert_allclose(cf["dk2"].sum(0), 0.0, atol=1e-12 * n)
+    np.testing.assert_allclose(cf["dv2"].sum(0), 0.0, atol=1e-12 * n)
+    # ... and a result with that property broken by a constant offset in P is caught by the same check
+    bad = closed_form(**x, scale=scale, causal=causal, lse=lse + 1e-3)
+    assert np.abs(bad["dv2"].sum(0)).max() > 1e-6
 
 
 def test_ddo_is_forward_jvp():

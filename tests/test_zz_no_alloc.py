@@ -19,8 +19,8 @@ def _plan(x, scale, causal):
     plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], scale, causal=causal,
                       impl="bf16", split=False)
     # a caller-owned workspace exactly as large as the library's array: same split decisions in both entry points
-    plan.ws_all = torch.empty(_lib.STATIC_WS_BYTES // 4, dtype=torch.float32, device="cuda")
-    plan.args.ws, plan.args.ws_bytes = plan.ws_all.data_ptr(), _lib.STATIC_WS_BYTES
+    plan.ws_all = torch.empty(_lib.lib().fhog_static_ws_bytes() // 4, dtype=torch.float32, device="cuda")
+    plan.args.ws, plan.args.ws_bytes = plan.ws_all.data_ptr(), _lib.lib().fhog_static_ws_bytes()
     return plan
 
 
@@ -67,7 +67,7 @@ def test_static_workspace_entry_point_rejects_what_does_not_fit():
     require_gpu()
     from fhog import _lib
     L = _lib.lib()
-    rows_max = _lib.STATIC_WS_BYTES // 12
+    rows_max = _lib.lib().fhog_static_ws_bytes() // 12
     x = with_caches(make_case(1, 128, 128, 64, torch.bfloat16, seed=32, grad_std=0.1), 0.125, False)
     from fhog import BwdBwdPlan
     plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125)
@@ -76,5 +76,34 @@ def test_static_workspace_entry_point_rejects_what_does_not_fit():
     rc = L.fhog_bwdbwd_static_ws(ctypes.byref(plan.args), None)
     assert rc == -2, rc
     msg = L.fhog_last_error().decode()
-    assert "static workspace" in msg and str(_lib.STATIC_WS_BYTES) in msg
+    assert "static workspace" in msg and str(_lib.lib().fhog_static_ws_bytes()) in msg
     assert L.fhog_bwdbwd_static_ws(None, None) == -1
+
+
+def test_static_workspace_entry_point_under_hip_graph_capture():
+    """One eager call first (it looks the array's address up and raises the kernels' LDS limit, neither of which may
+    run under capture), then the entry point is captured into a HIP graph and replayed: every replay gives the bits of
+    the eager call, with the program's own eager work and synchronisations in between."""
+    require_gpu()
+    from fhog import _lib
+    L = _lib.lib()
+    x = with_caches(make_case(4, 512, 512, 128, torch.bfloat16, seed=33, grad_std=0.1), 128 ** -0.5, True)
+    plan = _plan(x, 128 ** -0.5, True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _lib.check(L.fhog_bwdbwd_static_ws(ctypes.byref(plan.args), ctypes.c_void_p(side.cuda_stream)))   # warm-up, eager
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = [o.clone() for o in plan.outs]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(L.fhog_bwdbwd_static_ws(ctypes.byref(plan.args), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    for rep in range(3):
+        for o in plan.outs:
+            o.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("dq2", "dk2", "dv2", "ddo"), plan.outs, eager):
+            assert torch.equal(got, ref), (rep, name)
+        _ = (x["Q"].float() @ x["K"].float().transpose(-1, -2)).sum().item()   # unrelated eager work between replays
