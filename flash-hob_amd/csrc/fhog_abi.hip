@@ -60,7 +60,7 @@ int validate(const fhog_bwdbwd_args* a) {
     return fail(FHOG_E_DTYPE, "unknown dtype %d", a->dtype);
   if (a->impl != FHOG_IMPL_AUTO && a->impl != FHOG_IMPL_FP32 && a->impl != FHOG_IMPL_BF16)
     return fail(FHOG_E_IMPL, "unknown impl %d", a->impl);
-  if (a->schedule != FHOG_SCHEDULE_FOUR_PASS && a->schedule != FHOG_SCHEDULE_FUSED_STATS)
+  if (a->schedule < FHOG_SCHEDULE_FOUR_PASS || a->schedule > FHOG_SCHEDULE_THREE_SWEEP)
     return fail(FHOG_E_SCHEDULE, "unknown schedule %d", a->schedule);
   if (a->batch < 1 || a->n_q < 1 || a->n_k < 1)
     return fail(FHOG_E_SHAPE, "batch, n_q, n_k must be >= 1 (got %lld, %lld, %lld)", (long long)a->batch, (long long)a->n_q,
@@ -146,7 +146,7 @@ size_t split_bytes(const fhog_bwdbwd_args* a, int pass) {
 }
 // Splits a pass would like: enough workgroups for two per CU, every split keeping at least 8 streamed tiles.
 int wanted_split(const fhog_bwdbwd_args* a, int impl, int pass) {
-  if (impl != FHOG_IMPL_BF16 || pass == FHOG_PASS_D) return 1;
+  if (impl != FHOG_IMPL_BF16 || pass == FHOG_PASS_D || pass > FHOG_PASS_DD_B) return 1;   // passes 6-8 never split
   const bool kside = pass == FHOG_PASS_DK_DV;
   const int64_t groups = ((kside ? a->n_k : a->n_q) + 127) / 128 * a->batch;
   const int64_t streamed = ((kside ? a->n_q : a->n_k) + 31) / 32;
@@ -174,6 +174,8 @@ int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& base, int impl, int 
     p.tile_major = 0;
   p.part = reinterpret_cast<float*>(reinterpret_cast<char*>(a->ws) + stats_bytes(a));
   hipError_t e;
+  if (pass > FHOG_PASS_DD_B && impl != FHOG_IMPL_BF16)
+    return fail(FHOG_E_PASS, "pass %d exists in the 16-bit MFMA family only (bf16 / fp16 tensors, d in {64, 128})", pass);
   if (pass == FHOG_PASS_D)
     e = fhog::launch_rowdot(p, a->dtype, s);
   else if (impl == FHOG_IMPL_BF16)
@@ -379,7 +381,7 @@ int fhog_select_impl(const fhog_bwdbwd_args* args) {
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream) {
   const int rc = validate(args);
   if (rc != FHOG_OK) return rc;
-  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DD_B) return fail(FHOG_E_PASS, "unknown pass %d", pass);
+  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DD_B_DDO) return fail(FHOG_E_PASS, "unknown pass %d", pass);
   const fhog::Params p = to_params(args);
   return run_pass(args, p, select_impl(args), pass, (hipStream_t)hip_stream);
 }
@@ -389,13 +391,19 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   if (rc != FHOG_OK) return rc;
   const fhog::Params p = to_params(args);
   const int impl = select_impl(args);
-  const int four[] = {FHOG_PASS_D, FHOG_PASS_DD, FHOG_PASS_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
-  const int fused[] = {FHOG_PASS_D, FHOG_PASS_DD_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
-  const bool is_fused = args->schedule == FHOG_SCHEDULE_FUSED_STATS;
-  const int* order = is_fused ? fused : four;
-  const int n_pass = is_fused ? 4 : 5;
-  // the first statistics sweep of the 16-bit family writes d_i itself: no separate launch for it
-  for (int i = impl == FHOG_IMPL_BF16 ? 1 : 0; i < n_pass; i++) {
+  // Pass sequences. The first statistics sweep of the 16-bit family writes d_i itself: no separate launch for it there.
+  // The schedules that take ddO out of the third sweep exist in the 16-bit family; the fp32-MFMA family runs the
+  // reference's four passes for them.
+  static const int four[] = {FHOG_PASS_D, FHOG_PASS_DD, FHOG_PASS_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
+  static const int fused[] = {FHOG_PASS_D, FHOG_PASS_DD_B, FHOG_PASS_DQ_DDO, FHOG_PASS_DK_DV};
+  static const int ddo_early[] = {FHOG_PASS_DD, FHOG_PASS_B_DDO, FHOG_PASS_DQ, FHOG_PASS_DK_DV};
+  static const int three[] = {FHOG_PASS_DD_B_DDO, FHOG_PASS_DQ, FHOG_PASS_DK_DV};
+  const int* order = four;
+  int first = impl == FHOG_IMPL_BF16 ? 1 : 0, n_pass = 5;
+  if (args->schedule == FHOG_SCHEDULE_FUSED_STATS) order = fused, n_pass = 4;
+  if (args->schedule == FHOG_SCHEDULE_DDO_EARLY && impl == FHOG_IMPL_BF16) order = ddo_early, first = 0, n_pass = 4;
+  if (args->schedule == FHOG_SCHEDULE_THREE_SWEEP && impl == FHOG_IMPL_BF16) order = three, first = 0, n_pass = 3;
+  for (int i = first; i < n_pass; i++) {
     const int r = run_pass(args, p, impl, order[i], (hipStream_t)hip_stream);
     if (r != FHOG_OK) return r;
   }

@@ -70,6 +70,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int ROWS = 32 * NW;
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
+  // PASS 7 is pass 3 without its ddO half (dQ2 alone, for the schedules whose earlier sweep already produced ddO)
+  constexpr bool P3 = PASS == 3 || PASS == 7, WITH_DDO = PASS == 3;
   constexpr int TILE = TS * 2 * D;
   constexpr int STAGE = NT * TILE;
   constexpr int KK = D / 16;
@@ -118,7 +120,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   const float l_log2 = p.lse[row] * kLog2e;
   const float c_scale_log2 = p.scale * kLog2e;
   float dsum = 0.f;
-  if (PASS == 2 || PASS == 3) {
+  if (PASS == 2 || P3) {
     dsum = p.ws_d[row];
   } else {
     // The first statistics sweep of a chain also produces d_i = sum_c O_ic dO_ic (fhog/triton_bwdbwd.py:580) for the
@@ -133,8 +135,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
     dsum += __shfl_xor(dsum, 32);
     if (h == 0 && qi < p.n_q && split == 0) p.ws_d[row] = dsum;
   }
-  const float dd = (PASS == 2 || PASS == 3) ? p.ws_dd[row] : 0.f;
-  const float b = PASS == 3 ? p.ws_b[row] : 0.f;
+  const float dd = (PASS == 2 || P3) ? p.ws_dd[row] : 0.f;
+  const float b = P3 ? p.ws_b[row] : 0.f;
   const float kc = __builtin_fmaf(dd, dsum, b);   // per-row constant of dP' = E + (ddS - dd)(dP - d) - kc (passes 2, 3)
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
   // PASS 3 (d = 64): the second-level products follow in the same wave, with the S-shaped tiles as B operands
@@ -142,7 +144,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   constexpr int NC = D / 32;
   f32x16_t acc_dq[NC], acc_ddo[NC];
   int troff[NC][2];
-  if (PASS == 3) {
+  if (P3) {
 #pragma unroll
     for (int cb = 0; cb < NC; cb++) {
       acc_dq[cb] = f32x16_t{0};
@@ -215,7 +217,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
         } else if (ph == 2) {
           dds = mfma<F16>(a[c], Qb[kk], dds);
-          if (PASS == 3 && kk == 0 && masked) {
+          if (P3 && kk == 0 && masked) {
             keep_branch();
 #pragma unroll
             for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
@@ -224,7 +226,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 1) {
               pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
-            } else if (PASS == 3) {
+            } else if (P3) {
               dp[r] -= dsum;                           // u
               us[r] = pv[r] * dp[r];                   // dS = P u (scale applied to the accumulator at the end)
             } else if (PASS == 5) {
@@ -233,7 +235,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
           }
         } else {
           e = mfma<F16>(a[c], dOb[kk], e);
-          if (PASS != 3 && kk == 0 && masked) {
+          if (!P3 && kk == 0 && masked) {
             keep_branch();
 #pragma unroll
             for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
@@ -242,15 +244,15 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
           for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
             if (PASS == 2) {
               red = __builtin_fmaf(pv[r] * __builtin_fmaf(dds[r], p.scale, -dd), dp[r], red);   // P w u
-            } else if (PASS == 3) {
+            } else if (P3) {
               const float w = __builtin_fmaf(dds[r], p.scale, -dd);
               const float ddp = pv[r] * w;
               tt[r] = pv[r] * __builtin_fmaf(w, dp[r], -kc);   // z = P (w u - kc)
               if (r & 1) {
-                pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
+                if (WITH_DDO) pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
                 pk_ds[r / 2] = pack2<F16>(us[r - 1], us[r]);
-                pk_p[r / 2] = pack2<F16>(pv[r - 1], pv[r]);
-              } else {
+                if (WITH_DDO) pk_p[r / 2] = pack2<F16>(pv[r - 1], pv[r]);
+              } else if (WITH_DDO) {
                 dds[r] = ddp;
               }
             } else {
@@ -273,7 +275,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       } else if (PASS == 2) {
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
-      } else if (PASS == 3) {
+      } else if (P3) {
 #pragma unroll
         for (int r = 0; r < 16; r += 2)
           pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], tt[r]), __builtin_fmaf(pv[r + 1], e[r + 1], tt[r + 1]));
@@ -282,24 +284,54 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
         const auto opnd = [](const uint32_t* pk, int t) {
           return __builtin_bit_cast(bf16x8_t, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]});
         };
-        bf16x8_t ta[2][4];
+        constexpr int NX = WITH_DDO ? 4 : 2;   // staged tensors the second level reads: K, ddK (, V, ddV)
+        bf16x8_t ta[2][NX];
 #pragma unroll
-        for (int x = 0; x < 4; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+        for (int x = 0; x < NX; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+        if (WITH_DDO) {
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-          const int t = it / NC, cb = it % NC, c = it & 1;
-          if (it + 1 < NIT) {
-            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+          for (int it = 0; it < NIT; it++) {
+            const int t = it / NC, cb = it % NC, c = it & 1;
+            if (it + 1 < NIT) {
+              const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
 #pragma unroll
-            for (int x = 0; x < 4; x++)
-              ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+              for (int x = 0; x < NX; x++)
+                ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            acc_dq[cb] = mfma<F16>(ta[c][1], opnd(pk_ds, t), acc_dq[cb]);
+            acc_ddo[cb] = mfma<F16>(ta[c][NX - 2], opnd(pk_ddp, t), acc_ddo[cb]);
+            acc_dq[cb] = mfma<F16>(ta[c][0], opnd(pk_ds2, t), acc_dq[cb]);
+            acc_ddo[cb] = mfma<F16>(ta[c][NX - 1], opnd(pk_p, t), acc_ddo[cb]);
+            __builtin_amdgcn_sched_barrier(0);
           }
-          __builtin_amdgcn_sched_barrier(0);
-          acc_dq[cb] = mfma<F16>(ta[c][1], opnd(pk_ds, t), acc_dq[cb]);
-          acc_ddo[cb] = mfma<F16>(ta[c][2], opnd(pk_ddp, t), acc_ddo[cb]);
-          acc_dq[cb] = mfma<F16>(ta[c][0], opnd(pk_ds2, t), acc_dq[cb]);
-          acc_ddo[cb] = mfma<F16>(ta[c][3], opnd(pk_p, t), acc_ddo[cb]);
-          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          // dQ2 alone: two column blocks per round, so that the MFMAs on one accumulator are two instructions apart
+          constexpr int NP = NC / 2;
+          bf16x8_t tb[2][2][2];   // [buffer][column block of the pair][K | ddK]
+          const auto read_tb = [&](int buf, int it) {
+            const int t1 = it / NP, cp1 = it % NP;
+#pragma unroll
+            for (int cl = 0; cl < 2; cl++)
+#pragma unroll
+              for (int x = 0; x < 2; x++)
+                tb[buf][cl][x] = lds_read_tr_pre(stage + troff[2 * cp1 + cl][0], stage + troff[2 * cp1 + cl][1], x * TILE + t1 * 16 * 2 * D);
+          };
+#pragma unroll
+          for (int x = 0; x < 2; x++) tb[0][0][x] = ta[0][x];
+#pragma unroll
+          for (int x = 0; x < 2; x++) tb[0][1][x] = lds_read_tr_pre(stage + troff[1][0], stage + troff[1][1], x * TILE);
+#pragma unroll
+          for (int it = 0; it < 2 * NP; it++) {
+            const int t = it / NP, cp = it % NP, c = it & 1;
+            if (it + 1 < 2 * NP) read_tb(c ^ 1, it + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            acc_dq[2 * cp] = mfma<F16>(tb[c][0][1], opnd(pk_ds, t), acc_dq[2 * cp]);
+            acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][1], opnd(pk_ds, t), acc_dq[2 * cp + 1]);
+            acc_dq[2 * cp] = mfma<F16>(tb[c][0][0], opnd(pk_ds2, t), acc_dq[2 * cp]);
+            acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][0], opnd(pk_ds2, t), acc_dq[2 * cp + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       } else {
 #pragma unroll
@@ -309,7 +341,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
     dma_wait();
     __syncthreads();
   }
-  if (PASS == 3 && p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]
+  if (WITH_DDO && p.n_split > 1) {   // fp32 partial rows [split][dQ2 | ddO][batch * n_q][D]
     if (qi >= p.n_q) return;
     const int64_t rows = (int64_t)p.batch * p.n_q;
     float* pq = p.part + ((int64_t)split * 2 * rows + (int64_t)bh * p.n_q + qi) * D;
@@ -325,7 +357,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       }
     return;
   }
-  if (PASS == 3) {
+  if (P3) {
     if (qi >= p.n_q) return;
     uint16_t* odq = (uint16_t*)p.dq2 + qoff + (int64_t)qi * p.stride_qn;
     uint16_t* oddo = (uint16_t*)p.ddo + qoff + (int64_t)qi * p.stride_qn;
@@ -337,7 +369,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
         const f32x16_t& y = acc_ddo[cb];
         *reinterpret_cast<u32x2_t*>(odq + 32 * cb + 8 * g + 4 * h) =
             pack4<F16>(x[4 * g] * p.scale, x[4 * g + 1] * p.scale, x[4 * g + 2] * p.scale, x[4 * g + 3] * p.scale);
-        *reinterpret_cast<u32x2_t*>(oddo + 32 * cb + 8 * g + 4 * h) = pack4<F16>(y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]);
+        if (WITH_DDO) *reinterpret_cast<u32x2_t*>(oddo + 32 * cb + 8 * g + 4 * h) = pack4<F16>(y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]);
       }
     return;
   }
@@ -791,6 +823,13 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
         return hipErrorInvalidValue;
       }
       break;
+    case FHOG_PASS_DQ:
+      if constexpr (D == 64) {
+        e = launch_sweep<q_sweep_bf16<F16, D, 7, MASK>>(gq, 2 * 4 * tile, s, p);
+      } else {
+        return hipErrorInvalidValue;
+      }
+      break;
     case FHOG_PASS_DK_DV:
       if constexpr (D == 64) {
         e = launch_sweep<k_sweep_bf16<F16, D, MASK>>(gk, 2 * (3 * tile + 4 * TS * 4), s, p);
@@ -809,6 +848,7 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
 }  // namespace
 
 hipError_t launch_bf16_pc_pass(const Params& p, int pass, hipStream_t s);
+hipError_t launch_bf16_ddo_pass(const Params& p, int pass, hipStream_t s);
 
 bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
   (void)causal;
@@ -817,6 +857,8 @@ bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal) {
 
 hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
   if (!bf16_shape_supported(p.n_q, p.n_k, p.d, p.causal)) return hipErrorInvalidValue;
+  if (pass == FHOG_PASS_B_DDO || pass == FHOG_PASS_DD_B_DDO) return launch_bf16_ddo_pass(p, pass, s);
+  if (pass == FHOG_PASS_DQ && p.d == 128) return launch_bf16_pc_pass(p, pass, s);
   // d = 128: passes 3 and 4 need the producer/consumer split to fit the registers; d = 64: single-role kernels throughout
   if (p.d == 128 && (pass == FHOG_PASS_DQ_DDO || pass == FHOG_PASS_DK_DV)) {
     const hipError_t e = launch_bf16_pc_pass(p, pass, s);
@@ -831,7 +873,7 @@ hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
     else hipLaunchKernelGGL((combine_out<false, 128>), grid, dim3(256), 0, s, p.part, p.n_split, p.batch, n, sb, sn, out0, out1, p.scale);
     return hipGetLastError();
   }
-  if (pass < FHOG_PASS_DD || pass > FHOG_PASS_DD_B) return hipErrorInvalidValue;
+  if (pass < FHOG_PASS_DD || pass > FHOG_PASS_DQ || pass == FHOG_PASS_B_DDO) return hipErrorInvalidValue;
   const int mask = mask_mode(p);
 #define FHOG_SINGLE(F, DD)                                                             \
   (mask == MASK_NONE ? launch_single_d<F, DD, MASK_NONE>(p, pass, s)                   \

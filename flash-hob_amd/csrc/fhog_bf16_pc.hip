@@ -59,7 +59,8 @@ __device__ __forceinline__ void sop_write_pk(char* tile, const uint32_t* pk, int
 // ddV). KSIDE = true: pass 4 with the same stream: stationary rows = keys (rs = K, rdds = ddK, rdp = V, re = ddV),
 // streamed Q, dO, ddQ, dO again; the resident operand goes first in the MFMA, so that a lane still owns one QUERY (a
 // streamed row) and the row statistics stay per-lane scalars, reloaded for every tile; registers run over the keys.
-template <bool F16, int D, bool KSIDE>
+// DQ_ONLY (pass 3 without its ddO half, FHOG_PASS_DQ): ddP and P are not handed over.
+template <bool F16, int D, bool KSIDE, bool DQ_ONLY = false>
 __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf16x8_t* rs, const bf16x8_t* rdds,
                                           const bf16x8_t* rdp, const bf16x8_t* re, int lane, int lo, int hi, bool mask,
                                           float c_scale_log2, float l_log2, float scale, float dsum, float dd, float b) {
@@ -113,12 +114,12 @@ __device__ __forceinline__ void produce_q(const char* stage, char* sop, const bf
 #pragma unroll
       for (int r = EPK * kk; r < EPK * (kk + 1); r += 2) {
         const float ddp0 = pv[r] * __builtin_fmaf(dds[r], scale, -dd), ddp1 = pv[r + 1] * __builtin_fmaf(dds[r + 1], scale, -dd);
-        pk_ddp[r / 2] = pack2<F16>(ddp0, ddp1);
-        pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
+        if (!DQ_ONLY) pk_ddp[r / 2] = pack2<F16>(ddp0, ddp1);
+        if (!DQ_ONLY && !KSIDE) pk_p[r / 2] = pack2<F16>(pv[r], pv[r + 1]);
         z[r] = ddp0 * dp[r];
         z[r + 1] = ddp1 * dp[r + 1];
       }
-      if ((EPK * (kk + 1)) % 8 == 0) {
+      if (!DQ_ONLY && (EPK * (kk + 1)) % 8 == 0) {
         sop_write_pk(sop + 2 * SOP_TILE, pk_ddp, (EPK * kk) / 8, lane);
         if (!KSIDE) sop_write_pk(sop + 3 * SOP_TILE, pk_p, (EPK * kk) / 8, lane);   // pass 4 has no use for P
       }
@@ -255,7 +256,90 @@ __device__ __forceinline__ void consume_q(const Params& p, char* smem, const Str
       }
 }
 
+// Consumer wave of the dQ2-only sweep (FHOG_PASS_DQ): dQ2 = dS ddK + dS' K for the 32 queries of producer wave wq and
+// all D columns (D / 32 accumulators), from the operand tiles dS, dS' of that producer and the staged K and ddK.
 template <bool F16, int D, int MASK>
+__device__ __forceinline__ void consume_dq(const Params& p, char* smem, const StreamKeys<MASK>& geo, int j_begin, int j_end,
+                                           int q0, int wq, int lane, int bh) {
+  using SM = PCSmem<D, false>;
+  constexpr int NC = D / 32, NP = NC / 2, NIT = 2 * NP;
+  const int n = lane & 31, h = lane >> 5;
+  const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
+  const __bf16* src[4] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
+                          (const __bf16*)p.ddv + koff};
+  f32x16_t acc[NC];
+  int troff[NC][2];
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++) {
+    acc[cb] = f32x16_t{0};
+    troff[cb][0] = tr_lane_off_acc<D>(cb, 0, lane);
+    troff[cb][1] = tr_lane_off_acc<D>(cb, 1, lane);
+  }
+  const int qw0 = q0 + 32 * wq;
+  const char* sop_wave = smem + SM::SOP_BASE + wq * SM::SOP_WAVE;
+  Dma<D> dma;
+  dma.init(p.stride_kn, wq, lane);
+  const uint32_t ring_lds = lds_addr(smem);
+  if (j_begin < j_end)
+    dma.template issue_all<4>(ring_lds, SM::TILE, src, (int64_t)j_begin * TS * p.stride_kn, wq, p.n_k - j_begin * TS);
+  dma_wait();
+  __syncthreads();
+  int sc = RING - 1, sn = 1;  // ring slots of tile j-1 (read here) and tile j+1 (filled here)
+  for (int j = j_begin; j <= j_end; j++) {
+    if (j + 1 < j_end) {
+      const uint32_t dst = ring_lds + sn * SM::STAGE;
+      dma.template issue_all<4>(dst, SM::TILE, src, (int64_t)(j + 1) * TS * p.stride_kn, wq, p.n_k - (j + 1) * TS);
+    }
+    if (j > j_begin && !geo.dead((j - 1) * TS, qw0)) {   // block j-1 took part
+      const char* stage = smem + sc * SM::STAGE;
+      const char* sop = sop_wave + ((j - 1) & 1) * SM::SOP_BUF;
+      bf16x8_t bop[2][2][2];   // [buffer][column block of the pair][ddK | K]
+      bf16x8_t a_op[2][2];     // [k-step][dS | dS']
+      const auto read_b = [&](int buf, int it) {
+        const int t = it / NP, cp = it % NP;
+#pragma unroll
+        for (int cl = 0; cl < 2; cl++) {
+          const char* b0 = stage + troff[2 * cp + cl][0];
+          const char* b1 = stage + troff[2 * cp + cl][1];
+          bop[buf][cl][0] = lds_read_tr_pre(b0, b1, 1 * SM::TILE + t * 16 * 2 * D);
+          bop[buf][cl][1] = lds_read_tr_pre(b0, b1, 0 * SM::TILE + t * 16 * 2 * D);
+        }
+      };
+      read_b(0, 0);
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        a_op[t][0] = sop_read(sop + 0 * SOP_TILE, t, lane);
+        a_op[t][1] = sop_read(sop + 1 * SOP_TILE, t, lane);
+      }
+#pragma unroll
+      for (int it = 0; it < NIT; it++) {
+        const int t = it / NP, cp = it % NP, c = it & 1;
+        if (it + 1 < NIT) read_b(c ^ 1, it + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pr = 0; pr < 2; pr++)
+#pragma unroll
+          for (int cl = 0; cl < 2; cl++) acc[2 * cp + cl] = mfma<F16>(a_op[t][pr], bop[c][cl][pr], acc[2 * cp + cl]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    dma_wait();
+    __syncthreads();
+    sc = (sc == RING - 1) ? 0 : sc + 1;
+    sn = (sn == RING - 1) ? 0 : sn + 1;
+  }
+  // acc[cb][r] holds (query qw0 + 8*(r/4) + 4h + r%4, column 32 cb + n)
+  uint16_t* o = (uint16_t*)p.dq2 + qoff;
+#pragma unroll
+  for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int qrow = qw0 + 8 * (r / 4) + 4 * h + (r % 4);
+      if (qrow < p.n_q) o[(int64_t)qrow * p.stride_qn + 32 * cb + n] = to_elem<F16>(acc[cb][r] * p.scale);
+    }
+}
+
+template <bool F16, int D, int MASK, bool DQ_ONLY = false>
 __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   using SM = PCSmem<D, false>;
@@ -298,14 +382,16 @@ __global__ void __launch_bounds__(PC_THREADS) q_sweep3_pc(Params p) {
         const bool masked = geo.partial(k0, qw);
         int lo = 0, hi = 0;  // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
         if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
-        produce_q<F16, D, false>(stage, sop, Qb, ddQb, dOb, dOb, lane, lo, hi, masked, c_scale_log2, l_log2, p.scale, dsum, dd, b);
+        produce_q<F16, D, false, DQ_ONLY>(stage, sop, Qb, ddQb, dOb, dOb, lane, lo, hi, masked, c_scale_log2, l_log2, p.scale, dsum, dd, b);
       }
       __syncthreads();
       sp = (sp == RING - 1) ? 0 : sp + 1;
     }
   } else {
+    // dQ2 alone: consumer wave wq owns the 32 queries of producer wave wq
+    if (DQ_ONLY) consume_dq<F16, D, MASK>(p, smem, geo, j_begin, j_end, q0, wq, lane, bh);
     // consumer wave (qp, out) owns the 64-query x D-column block of ONE output for the query pair qp
-    if (wq & 1) consume_q<F16, D, MASK, 1>(p, smem, geo, j_begin, j_end, q0, wq, lane, split, bh);
+    else if (wq & 1) consume_q<F16, D, MASK, 1>(p, smem, geo, j_begin, j_end, q0, wq, lane, split, bh);
     else consume_q<F16, D, MASK, 0>(p, smem, geo, j_begin, j_end, q0, wq, lane, split, bh);
   }
 }
@@ -747,7 +833,12 @@ template <bool F16, int D, int MASK>
 hipError_t launch_pc_d(const Params& p, int pass, hipStream_t s) {
   const dim3 block(PC_THREADS);
   hipError_t e;
-  if (pass == FHOG_PASS_DQ_DDO) {
+  if (pass == FHOG_PASS_DQ) {
+    const int smem = PCSmem<D, false>::TOTAL;
+    e = allow_dynamic_lds<q_sweep3_pc<F16, D, MASK, true>>(smem);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((q_sweep3_pc<F16, D, MASK, true>), dim3(grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch)), block, smem, s, p);
+  } else if (pass == FHOG_PASS_DQ_DDO) {
     const int smem = PCSmem<D, false>::TOTAL;
     e = allow_dynamic_lds<q_sweep3_pc<F16, D, MASK>>(smem);
     if (e != hipSuccess) return e;

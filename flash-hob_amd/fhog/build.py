@@ -16,7 +16,7 @@ PKG_DIR = Path(__file__).resolve().parent            # .../flash-hob_amd/fhog
 CSRC = PKG_DIR.parent / "csrc"
 INCLUDE = PKG_DIR.parent.parent / "include"
 LIB_PATH = PKG_DIR / "libfhog_hip.so"
-SOURCES = ["fhog_abi.hip", "fhog_fp32.hip", "fhog_bf16.hip", "fhog_bf16_pc.hip", "fhog_attn.hip", "fhog_attn_fp32.hip", "fhog_probe.hip"]
+SOURCES = ["fhog_abi.hip", "fhog_fp32.hip", "fhog_bf16.hip", "fhog_bf16_pc.hip", "fhog_bf16_ddo.hip", "fhog_attn.hip", "fhog_attn_fp32.hip", "fhog_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

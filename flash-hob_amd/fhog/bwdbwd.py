@@ -12,6 +12,19 @@ from . import _lib
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32, torch.float16: _lib.DTYPE_FP16}
 _IMPLS = {None: _lib.IMPL_AUTO, "auto": _lib.IMPL_AUTO, "fp32": _lib.IMPL_FP32, "bf16": _lib.IMPL_BF16}
+_SCHEDULES = {None: _lib.SCHEDULE_FOUR_PASS, "four_pass": _lib.SCHEDULE_FOUR_PASS, "fused_stats": _lib.SCHEDULE_FUSED_STATS,
+              "ddo_early": _lib.SCHEDULE_DDO_EARLY, "three_sweep": _lib.SCHEDULE_THREE_SWEEP}
+
+
+def schedule_code(schedule, fused_stats: bool = False) -> int:
+    """FHOG_SCHEDULE_* of the C ABI for the Python-level arguments (``fused_stats=True`` is ``schedule="fused_stats"``)."""
+    if schedule not in _SCHEDULES:
+        raise ValueError(f"schedule must be one of {sorted(k for k in _SCHEDULES if k)} or None, got {schedule!r}")
+    if fused_stats:
+        if schedule not in (None, "fused_stats"):
+            raise ValueError(f"fused_stats=True contradicts schedule={schedule!r}")
+        return _lib.SCHEDULE_FUSED_STATS
+    return _SCHEDULES[schedule]
 
 
 def _flatten(t: torch.Tensor, name: str) -> torch.Tensor:
@@ -84,7 +97,7 @@ def _workspace(args: "_lib.BwdBwdArgs", device, split: bool) -> torch.Tensor:
     return ws
 
 
-def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, fused_stats=False,
+def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws, schedule=0,
                 window=None) -> _lib.BwdBwdArgs:
     """``ws``: a workspace tensor of the minimum size, or None when :func:`_workspace` fills it in afterwards."""
     a = _lib.BwdBwdArgs()
@@ -101,13 +114,13 @@ def _build_args(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, causal, impl, outs, ws,
     a.dtype = _DTYPES[Q.dtype]
     a.causal, a.window = mask_code(causal, window, Q.shape[1], K.shape[1])
     a.impl = impl
-    a.schedule = 1 if fused_stats else 0
+    a.schedule = int(schedule)
     return a
 
 
 def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window: Optional[int] = None,
-                 impl: Optional[str] = None, fused_stats: bool = False, return_stats: bool = False, only_pass: Optional[int] = None,
-                 split: bool = True):
+                 impl: Optional[str] = None, fused_stats: bool = False, schedule: Optional[str] = None,
+                 return_stats: bool = False, only_pass: Optional[int] = None, split: bool = True):
     """Flash Higher-Order-Gradients: VJP of the attention backward pass.
 
     Same positional signature and return order as the reference
@@ -134,6 +147,11 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
         fused_stats: opt-in schedule that takes ``dd`` and ``b`` from one sweep instead of the reference's two
             (``fhog/triton_bwdbwd.py:185-251``): 22 instead of 25 recomputed products; ``b`` then differs from the
             default schedule's value only by fp32 summation order.
+        schedule: None / "four_pass" (the reference's four sweeps, 25 recomputed products) or one of the opt-in
+            schedules "fused_stats" (22), "ddo_early" (23: four sweeps, the second one yields ``ddO`` together with
+            ``b_i = dO_i . ddO_i - d_i dd_i``, the third ``dQ2`` alone) and "three_sweep" (20: ``dd``, ``b`` and ``ddO``
+            from one sweep, then ``dQ2``, then ``dK2`` and ``dV2``). The last two exist in the 16-bit kernels; fp32
+            tensors run the reference schedule whatever is asked.
         return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
         only_pass: run a single pass (0..5, see fhog._lib.PASS_*) instead of the whole chain; for tests and profiling.
         split: allocate the larger workspace that lets launches too small to fill the GPU split their streamed side over
@@ -175,6 +193,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
     if d not in (32, 64, 128):
         raise ValueError(f"head dim {d} not supported (32, 64 or 128)")
     mask_code(causal, window, n_q, n_k)  # raises on an inapplicable mask
+    sched = schedule_code(schedule, fused_stats)
     if not Q.is_cuda:
         raise ValueError("flash_bwdbwd runs on the GPU only: tensors must be on a ROCm device (there is no CPU path)")
     lse = L.reshape(batch, n_q)
@@ -190,7 +209,7 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
         dk2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
         dv2 = torch.empty_strided(k3.shape, k3.stride(), dtype=Q.dtype, device=Q.device)
         args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl],
-                           (dq2, dk2, dv2, ddo), None, fused_stats, window)
+                           (dq2, dk2, dv2, ddo), None, sched, window)
         ws = _workspace(args, Q.device, split)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         L_ = _lib.lib()
@@ -215,7 +234,7 @@ class BwdBwdPlan:
     """
 
     def __init__(self, Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, window=None, impl=None,
-                 fused_stats=False, split=True):
+                 fused_stats=False, schedule=None, split=True):
         ts = [_flatten(t, "tensor") for t in (Q, K, V, O, dO, ddQ, ddK, ddV)]
         q3, k3, v3, o3, do3, ddq3, ddk3, ddv3 = ts
         q3, o3, do3, ddq3 = _prepare_group([q3, o3, do3, ddq3], "q")
@@ -224,7 +243,7 @@ class BwdBwdPlan:
         lse = L.reshape(batch, n_q).to(torch.float32).contiguous()
         self.keep = (q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse)
         self.outs = (torch.empty_like(q3), torch.empty_like(k3), torch.empty_like(v3), torch.empty_like(q3))
-        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, None, fused_stats, window)
+        self.args = _build_args(q3, k3, v3, o3, do3, ddq3, ddk3, ddv3, lse, scale, causal, _IMPLS[impl], self.outs, None, schedule_code(schedule, fused_stats), window)
         with torch.cuda.device(Q.device):
             self.ws_all = _workspace(self.args, Q.device, split)   # d | dd | b, then partial results of split launches
         self.ws = self.ws_all[:3 * batch * n_q]

@@ -38,6 +38,11 @@ def pass_of(kernel):
     m = re.match(r"q_sweep_bf16<\w+, \d+, (\d)", kernel)
     if m:
         return int(m.group(1))
+    m = re.match(r"q_sweep_ddo<\w+, \d+, \d, (\w+)>", kernel)
+    if m:
+        return 6 if m.group(1) == "true" else 8
+    if re.match(r"q_sweep3_pc<\w+, \d+, \d, true>", kernel):
+        return 7
     for prefix, p in (("dd_sweep64_bf16", 1), ("q_sweep3_pc", 3), ("k_sweep_pc", 4), ("k_sweep_bf16", 4), ("rowdot", 0), ("attn_fwd", "fwd"),
                       ("attn_bwd_q", "bwd_q"), ("attn_bwd_k", "bwd_k")):
         if kernel.startswith(prefix):
@@ -50,7 +55,8 @@ def algorithmic_mib(w, p):
     es = w.dtype.itemsize
     qt, kt, rv = w.batch * w.n_q * w.d * es / 2 ** 20, w.batch * w.n_k * w.d * es / 2 ** 20, w.batch * w.n_q * 4 / 2 ** 20
     table = {0: (2 * qt, rv), 1: (4 * qt + 2 * kt + rv, 2 * rv), 2: (3 * qt + 4 * kt + 3 * rv, rv),
-             5: (4 * qt + 4 * kt + rv, 3 * rv), 3: (3 * qt + 4 * kt + 4 * rv, 2 * qt), 4: (3 * qt + 4 * kt + 4 * rv, 2 * kt),
+             5: (4 * qt + 4 * kt + rv, 3 * rv), 6: (3 * qt + 4 * kt + 3 * rv, qt + rv), 7: (3 * qt + 4 * kt + 4 * rv, qt),
+             8: (4 * qt + 4 * kt + rv, qt + 3 * rv), 3: (3 * qt + 4 * kt + 4 * rv, 2 * qt), 4: (3 * qt + 4 * kt + 4 * rv, 2 * kt),
              "fwd": (qt + 2 * kt, qt + rv), "bwd_q": (2 * qt + 2 * kt + 2 * rv, qt), "bwd_k": (2 * qt + 2 * kt + 2 * rv, 2 * kt)}
     return table.get(p)
 
@@ -116,10 +122,12 @@ def main():
     P("Commands (from the repository root on one MI355X):\n")
     P(COMMANDS.replace("W=cfg2_bf16_causal_4096_d128", f"W={w.name}"))
     P("""
-`bench.py --profile-only` runs the timed loop of the default four-pass schedule, then three calls of the opt-in
-fused-statistics schedule (pass 5 replaces passes 1 and 2), then three calls of the first-order kernels on the same tensors,
-then a streaming `torch.add` used to calibrate the byte counters. Template arguments of the kernels:
-`<fp16?, d, [pass,] mask mode[, waves per workgroup]>` (mask mode 1 = square causal mask).
+`bench.py --profile-only` runs the timed loop of the default four-pass schedule, then three calls each of the opt-in
+schedules (fused statistics: pass 5 replaces passes 1 and 2; ddO early: `q_sweep_ddo<.., true>` = pass 6 and
+`q_sweep3_pc<.., true>` = pass 7 replace passes 2 and 3; three sweeps: `q_sweep_ddo<.., false>` = pass 8, then pass 7),
+then three calls of the first-order kernels on the same tensors, then a streaming `torch.add` used to calibrate the byte
+counters. Template arguments of the kernels: `<fp16?, d, [pass,] mask mode[, waves per workgroup | variant]>` (mask mode
+1 = square causal mask).
 
 ## kernel-trace --stats (kt_kernel_stats.csv), library kernels only
 

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define FHOG_ABI_VERSION 4
+#define FHOG_ABI_VERSION 5
 
 /* element types of Q,K,V,O,dO,ddQ,ddK,ddV and of the four outputs */
 #define FHOG_DTYPE_BF16 0
@@ -61,6 +61,14 @@ extern "C" {
 #define FHOG_PASS_DD_B 5   /* passes 1 and 2 in one sweep: b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
                               (same quantities as fhog/triton_bwdbwd.py:185-251, three recomputed products fewer) */
 
+/* passes of the opt-in schedules that take ddO out of the third sweep (16-bit MFMA family; see FHOG_SCHEDULE_*) */
+#define FHOG_PASS_B_DDO 6    /* second sweep as S, ddS, P ddV, ddP V: writes ddO and b_i = dO_i . ddO_i - d_i dd_i (an
+                                identity of the reference's quantities: sum_j P_ij dP_ij = d_i); reads d, dd */
+#define FHOG_PASS_DQ 7       /* third sweep for dQ2 alone (ddO is already there): seven products instead of nine */
+#define FHOG_PASS_DD_B_DDO 8 /* passes 1 and 6 in one sweep: dd_i is accumulated next to (P ddV)_i and ((P o ddS) V)_i
+                                and taken out at the end of the row, ddO_i = ... - dd_i O_i (sum_j P_ij V_j = O_i);
+                                writes d, dd, b, ddO */
+
 /* kernel families (fhog_bwdbwd_args.impl) */
 #define FHOG_IMPL_AUTO 0   /* 16-bit MFMA kernels for bf16/fp16 tensors when the shape allows, else the fp32-MFMA kernels */
 #define FHOG_IMPL_FP32 1   /* force the fp32-MFMA kernels (any dtype; every intermediate in fp32) */
@@ -79,6 +87,15 @@ extern "C" {
                                        (fhog/triton_bwdbwd.py:185-313, 467-535); 25 recomputed products */
 #define FHOG_SCHEDULE_FUSED_STATS 1 /* opt-in: dd and b from one sweep (FHOG_PASS_DD_B), 22 recomputed products;
                                        b differs from the four-pass value only by fp32 summation order */
+#define FHOG_SCHEDULE_DDO_EARLY 2   /* opt-in, still four sweeps in the reference's order: dd; b together with ddO
+                                       (FHOG_PASS_B_DDO); dQ2 alone (FHOG_PASS_DQ); dK2+dV2. 23 recomputed products.
+                                       b inherits the 16-bit rounding of the P and ddP operands of ddO */
+#define FHOG_SCHEDULE_THREE_SWEEP 3 /* opt-in, three sweeps: dd, b and ddO (FHOG_PASS_DD_B_DDO); dQ2 (FHOG_PASS_DQ);
+                                       dK2+dV2. 20 recomputed products. ddP V is formed as (P o ddS) V - dd O with the
+                                       caller's 16-bit O: accurate as long as dd_i does not dominate ddS_ij - dd_i.
+                                       Schedules 2 and 3 exist in the 16-bit MFMA family; the fp32-MFMA family runs the
+                                       four-pass schedule for them, and launches too small to fill the GPU do not split
+                                       their streamed side in the passes 6, 7 and 8 */
 
 /* Launch choices (the counterpart of the reference's autotune list, fhog/triton_bwdbwd.py:12-36) are fixed functions of
  * the launch size. For experiments they can be overridden through the environment variable FHOG_TUNE, a comma-separated
