@@ -107,7 +107,7 @@ def test_attn_validate(L, mutate, backward, code, word):
 
 
 def test_version_and_workspace(L):
-    assert L.fhog_abi_version() == 4
+    assert L.fhog_abi_version() == 5
     assert L.fhog_bwdbwd_workspace_bytes(32, 4096) == 3 * 32 * 4096 * 4
     assert L.fhog_bwdbwd_workspace_bytes(-1, 5) == 0
 
