@@ -299,6 +299,7 @@ const Tuning& tuning() {
       if (!strcmp(tok, "b8")) flag(tok, val, &r.b8);
       else if (!strcmp(tok, "split")) flag(tok, val, &r.split);
       else if (!strcmp(tok, "dd64")) flag(tok, val, &r.dd64);
+      else if (!strcmp(tok, "stage64")) flag(tok, val, &r.stage64);
       else if (!strcmp(tok, "order")) {
         if (!strcmp(val, "tile")) r.order = 1;
         else if (!strcmp(val, "slice")) r.order = 0;

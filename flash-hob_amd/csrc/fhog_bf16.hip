@@ -65,7 +65,9 @@ __global__ void __launch_bounds__(256) combine_out(const float* part, int n_spli
   *reinterpret_cast<u32x2_t*>(out1 + o) = pack4<F16>(b[0], b[1], b[2], b[3]);
 }
 
-template <bool F16, int D, int PASS, int MASK, int NW = 4>
+// SUB: 32-row tiles staged and consumed per barrier. SUB = 2 is a 64-row stage: one barrier, one round of staging
+// issues and one set of stage addresses per two blocks (twice the LDS), for the head dim whose blocks are short.
+template <bool F16, int D, int PASS, int MASK, int NW = 4, int SUB = 1>
 __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int ROWS = 32 * NW;
@@ -108,8 +110,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   Dma<D> dma;
   dma.init(p.stride_kn, wave & 3, lane);
   const uint32_t ring_lds = lds_addr(smem) + half * NLD * TILE;
-  if (j_begin < j_end)
-    dma.template issue_all<NLD>(ring_lds + (j_begin & 1) * STAGE, TILE, srcl, (int64_t)j_begin * TS * p.stride_kn, wave & 3, p.n_k - j_begin * TS);
+  // the ring holds 2 * SUB tiles; tile j lives in slot (j - j_begin) mod (2 * SUB)
+  const auto stage_tile = [&](int j) {
+    const uint32_t dst = ring_lds + ((j - j_begin) & (2 * SUB - 1)) * STAGE;
+    dma.template issue_all<NLD>(dst, TILE, srcl, (int64_t)j * TS * p.stride_kn, wave & 3, p.n_k - j * TS);
+  };
+#pragma unroll
+  for (int u = 0; u < SUB; u++)
+    if (j_begin + u < j_end) stage_tile(j_begin + u);
 
   bf16x8_t Qb[KK], ddQb[KK], dOb[KK];
   load_resident<D>(Qb, (const __bf16*)p.q + qoff, p.stride_qn, qr, h);
@@ -165,18 +173,20 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   dma_wait();
   __syncthreads();
 
-  for (int j = j_begin; j < j_end; j++) {
-    if (j + 1 < j_end) {
-      const uint32_t dst = ring_lds + ((j + 1) & 1) * STAGE;
-      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_kn;
-      dma.template issue_all<NLD>(dst, TILE, srcl, adv, wave & 3, p.n_k - (j + 1) * TS);
-    }
+  for (int jj = j_begin; jj < j_end; jj += SUB) {
+#pragma unroll
+    for (int u = 0; u < SUB; u++)
+      if (jj + SUB + u < j_end) stage_tile(jj + SUB + u);
+#pragma unroll
+    for (int u = 0; u < SUB; u++) {
+    const int j = jj + u;
+    if (SUB > 1 && j >= j_end) continue;
     const int k0 = j * TS;
     const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
     int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
     if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
     if (!geo.dead(k0, qw)) {  // else every key of the tile is hidden from this wave
-      const char* stage = smem + (j & 1) * STAGE;
+      const char* stage = smem + (((jj - j_begin) & SUB) + u) * STAGE;
       // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
       // is cut into small pieces placed right behind the MFMAs of the same wave, where it runs in the
       // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
@@ -337,6 +347,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
 #pragma unroll
         for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], us[r] + e[r], red);
       }
+    }
     }
     dma_wait();
     __syncthreads();
@@ -552,7 +563,8 @@ __global__ void __launch_bounds__(256, 2) dd_sweep64_bf16(Params p) {
 // accumulator registers run over the queries; rounded to 16 bits they are the B operands of the second-level
 // products (contraction over the queries), whose A operands are transposing reads of the staged Q-side tiles.
 // At d = 64 everything fits 256 registers, so no S-shaped tile passes through LDS.
-template <bool F16, int D, int MASK>
+// SUB: 32-query tiles staged and consumed per barrier (see q_sweep_bf16).
+template <bool F16, int D, int MASK, int SUB = 1>
 __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D;
@@ -603,48 +615,62 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
   Dma<D> dma;
   dma.init(p.stride_qn, wave, lane);
   const uint32_t ring_lds = lds_addr(smem);
-  float stat_reg = 0.f, stat_d = 0.f, stat_dd = 0.f;
+  float stat_reg[SUB] = {}, stat_d[SUB] = {}, stat_dd[SUB] = {};   // one set per tile of a group
   // The statistic is loaded (a global, not generic, load) before the staging loads of a step and first touched at
   // the end of the step, so the wave never waits for it in between. Staged per query: L log2(e), -d, dd and
   // -(dd d + b), the values the accumulators of dP and E start from (the threads of the last group load d and dd too).
-  auto load_stat = [&](int q_base) {
+  auto load_stat = [&](int u, int q_base) {
     if (tid < 4 * TS) {
       const int q = min(q_base + (tid & (TS - 1)), p.n_q - 1);
-      stat_reg = *(global_f32_ptr)(stat_src + q);
+      stat_reg[u] = *(global_f32_ptr)(stat_src + q);
       if (tid >= 3 * TS) {
-        stat_d = *(global_f32_ptr)(p.ws_d + (int64_t)bh * p.n_q + q);
-        stat_dd = *(global_f32_ptr)(p.ws_dd + (int64_t)bh * p.n_q + q);
+        stat_d[u] = *(global_f32_ptr)(p.ws_d + (int64_t)bh * p.n_q + q);
+        stat_dd[u] = *(global_f32_ptr)(p.ws_dd + (int64_t)bh * p.n_q + q);
       }
     }
   };
-  auto store_stat = [&](char* stage_base) {
+  auto store_stat = [&](int u, char* stage_base) {
     if (tid < 4 * TS) {
       const int g = tid / TS;
       reinterpret_cast<float*>(stage_base + 3 * TILE)[tid] =
-          g == 0 ? stat_reg * kLog2e : g == 1 ? -stat_reg : g == 2 ? stat_reg : -__builtin_fmaf(stat_dd, stat_d, stat_reg);
+          g == 0 ? stat_reg[u] * kLog2e : g == 1 ? -stat_reg[u] : g == 2 ? stat_reg[u] : -__builtin_fmaf(stat_dd[u], stat_d[u], stat_reg[u]);
     }
   };
+  // the ring holds two groups of SUB tiles; tile j lives in slot (j - t_begin) mod (2 * SUB)
+  const auto stage_tile = [&](int j) {
+    const uint32_t dst = ring_lds + ((j - t_begin) & (2 * SUB - 1)) * STAGE;
+    dma.template issue_all<3>(dst, TILE, src, (int64_t)j * TS * p.stride_qn, wave, p.n_q - j * TS);
+  };
+#pragma unroll
+  for (int u = 0; u < SUB; u++)
+    if (t_begin + u < t_end) {
+      load_stat(u, (t_begin + u) * TS);
+      stage_tile(t_begin + u);
+    }
   if (t_begin < t_end) {
-    load_stat(t_begin * TS);
-    const int64_t adv = (int64_t)t_begin * TS * p.stride_qn;
-    dma.template issue_all<3>(ring_lds, TILE, src, adv, wave, p.n_q - t_begin * TS);
     wait_vm0();
-    store_stat(smem);
+#pragma unroll
+    for (int u = 0; u < SUB; u++)
+      if (t_begin + u < t_end) store_stat(u, smem + u * STAGE);
   }
   dma_wait();
   __syncthreads();
 
-  for (int j = t_begin; j < t_end; j++) {
-    const int st = (j - t_begin) & 1;
-    if (j + 1 < t_end) {
-      load_stat((j + 1) * TS);
-      const uint32_t dst = ring_lds + (st ^ 1) * STAGE;
-      const int64_t adv = (int64_t)(j + 1) * TS * p.stride_qn;
-      dma.template issue_all<3>(dst, TILE, src, adv, wave, p.n_q - (j + 1) * TS);
-    }
+  for (int jj = t_begin; jj < t_end; jj += SUB) {
+    const int grp = (jj - t_begin) & SUB;   // first ring slot of this group; the other group starts at grp ^ SUB
+#pragma unroll
+    for (int u = 0; u < SUB; u++)
+      if (jj + SUB + u < t_end) {
+        load_stat(u, (jj + SUB + u) * TS);
+        stage_tile(jj + SUB + u);
+      }
+#pragma unroll
+    for (int u = 0; u < SUB; u++) {
+    const int j = jj + u;
+    if (SUB > 1 && j >= t_end) continue;
     const int qb = j * TS;
     if (!geo.dead(qb, kw)) {  // else no query of the tile sees a key of this wave
-      const char* stage = smem + st * STAGE;
+      const char* stage = smem + (grp + u) * STAGE;
       const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
       // five first-level products in one stream of KK k-steps; the three staged operands of step kk + 1 are
       // fetched before the MFMAs of step kk: S = Q K^T, ddS = ddQ K^T + Q ddK^T, dP = dO V^T, E = dO ddV^T
@@ -727,9 +753,12 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if (j + 1 < t_end) {
+    }
+    if (jj + SUB < t_end) {
       wait_vm0();
-      store_stat(smem + (st ^ 1) * STAGE);
+#pragma unroll
+      for (int u = 0; u < SUB; u++)
+        if (jj + SUB + u < t_end) store_stat(u, smem + ((grp ^ SUB) + u) * STAGE);
     }
     dma_wait();
     __syncthreads();
@@ -800,22 +829,31 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
     if (pass == FHOG_PASS_DD && !split && (dd64 < 0 ? g8 >= 2048 : dd64 == 1))
       return launch_sweep<dd_sweep64_bf16<F16, D, MASK>>(g8, 2 * 2 * tile, s, p, 256);
   }
+  // d = 64: a block is half as long as at d = 128 while the work per barrier, staging issue and set of stage addresses
+  // stays, so the sweeps stage and consume two 32-row tiles per barrier (SUB = 2, twice the LDS); FHOG_TUNE stage64=0
+  // keeps one.
+  constexpr int S2 = D == 64 ? 2 : 1;
+  const bool two = D == 64 && tuning().stage64 != 0;
   switch (pass) {
     case FHOG_PASS_DD:
-      e = launch_sweep<q_sweep_bf16<F16, D, 1, MASK>>(gq, 2 * 2 * tile, s, p);
+      e = two ? launch_sweep<q_sweep_bf16<F16, D, 1, MASK, 4, S2>>(gq, 2 * S2 * 2 * tile, s, p)
+              : launch_sweep<q_sweep_bf16<F16, D, 1, MASK>>(gq, 2 * 2 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<1>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_B:
-      e = launch_sweep<q_sweep_bf16<F16, D, 2, MASK>>(gq, 2 * 4 * tile, s, p);
+      e = two ? launch_sweep<q_sweep_bf16<F16, D, 2, MASK, 4, S2>>(gq, 2 * S2 * 4 * tile, s, p)
+              : launch_sweep<q_sweep_bf16<F16, D, 2, MASK>>(gq, 2 * 4 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<2>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_DD_B:
-      e = launch_sweep<q_sweep_bf16<F16, D, 5, MASK>>(gq, 2 * 4 * tile, s, p);
+      e = two ? launch_sweep<q_sweep_bf16<F16, D, 5, MASK, 4, S2>>(gq, 2 * S2 * 4 * tile, s, p)
+              : launch_sweep<q_sweep_bf16<F16, D, 5, MASK>>(gq, 2 * 4 * tile, s, p);
       if (e == hipSuccess && split) hipLaunchKernelGGL(combine_stats<5>, dim3((unsigned)((rows_q + 255) / 256)), dim3(256), 0, s, p);
       break;
     case FHOG_PASS_DQ_DDO:
       if constexpr (D == 64) {
-        e = launch_sweep<q_sweep_bf16<F16, D, 3, MASK>>(gq, 2 * 4 * tile, s, p);
+        e = two ? launch_sweep<q_sweep_bf16<F16, D, 3, MASK, 4, S2>>(gq, 2 * S2 * 4 * tile, s, p)
+                : launch_sweep<q_sweep_bf16<F16, D, 3, MASK>>(gq, 2 * 4 * tile, s, p);
         if (e == hipSuccess && split)
           hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_q * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
                              p.batch, p.n_q, p.stride_qb, p.stride_qn, (uint16_t*)p.dq2, (uint16_t*)p.ddo, p.scale);
@@ -825,14 +863,16 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
       break;
     case FHOG_PASS_DQ:
       if constexpr (D == 64) {
-        e = launch_sweep<q_sweep_bf16<F16, D, 7, MASK>>(gq, 2 * 4 * tile, s, p);
+        e = two ? launch_sweep<q_sweep_bf16<F16, D, 7, MASK, 4, S2>>(gq, 2 * S2 * 4 * tile, s, p)
+                : launch_sweep<q_sweep_bf16<F16, D, 7, MASK>>(gq, 2 * 4 * tile, s, p);
       } else {
         return hipErrorInvalidValue;
       }
       break;
     case FHOG_PASS_DK_DV:
       if constexpr (D == 64) {
-        e = launch_sweep<k_sweep_bf16<F16, D, MASK>>(gk, 2 * (3 * tile + 4 * TS * 4), s, p);
+        e = two ? launch_sweep<k_sweep_bf16<F16, D, MASK, S2>>(gk, 2 * S2 * (3 * tile + 4 * TS * 4), s, p)
+                : launch_sweep<k_sweep_bf16<F16, D, MASK>>(gk, 2 * (3 * tile + 4 * TS * 4), s, p);
         if (e == hipSuccess && split)
           hipLaunchKernelGGL((combine_out<F16, D>), dim3((unsigned)((rows_k * (D / 4) + 255) / 256)), dim3(256), 0, s, p.part, p.n_split,
                              p.batch, p.n_k, p.stride_kb, p.stride_kn, (uint16_t*)p.dk2, (uint16_t*)p.dv2, p.scale);

@@ -12,8 +12,10 @@
 //                       (FHOG_PASS_DD_B_DDO; it also writes d_i = O_i . dO_i for the sweeps behind it)
 //
 // Single-role kernel of the shape of the statistics sweeps: 256 threads = 4 wave64 own 128 queries, two workgroups per
-// CU; a wave keeps Q and ddQ of its 32 queries in registers as MFMA B operands; K, ddK, V, ddV stream through a
-// two-stage LDS ring of 32-key tiles filled by direct global->LDS loads. First-level products have the keys as M and
+// CU (NW = 8: 512 threads own 256 queries, one workgroup per CU, for launches with plenty of workgroups: every staged
+// tile then serves twice the rows, i.e. half the staging loads per row). A wave keeps Q and ddQ of its 32 queries in
+// registers as MFMA B operands; K, ddK, V, ddV stream through a two-stage LDS ring of 32-key tiles filled by direct
+// global->LDS loads. First-level products have the keys as M and
 // the queries as N, so a lane owns one query; P and ddP, rounded to 16 bits, are the B operands of the second-level
 // products as they stand in the registers (contraction over the keys), whose A operands are transposing reads of the
 // staged V and ddV tiles: nothing S-shaped passes through LDS, and one 32 x D fp32 accumulator (ddO^T: lane = query,
@@ -24,17 +26,17 @@ namespace fhog {
 using namespace bf16k;
 namespace {
 
-template <bool F16, int D, int MASK, bool KNOWN_DD>
-__global__ void __launch_bounds__(256, 2) q_sweep_ddo(Params p) {
+template <bool F16, int D, int MASK, bool KNOWN_DD, int NW = 4>
+__global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_ddo(Params p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  constexpr int NT = 4, TILE = TS * 2 * D, STAGE = NT * TILE, KK = D / 16, NC = D / 32;
+  constexpr int NT = 4, TILE = TS * 2 * D, STAGE = NT * TILE, KK = D / 16, NC = D / 32, ROWS = 32 * NW;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
+  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
-  const int q0 = tile * WG_ROWS, qw = q0 + 32 * wave, qi = qw + n;
+  const int q0 = tile * ROWS, qw = q0 + 32 * wave, qi = qw + n;
   const int qr = min(qi, p.n_q - 1);  // queries past the end compute on a copy of the last row and store nothing
   const int64_t qoff = (int64_t)bh * p.stride_qb, koff = (int64_t)bh * p.stride_kb;
   const __bf16* src[NT] = {(const __bf16*)p.k + koff, (const __bf16*)p.ddk + koff, (const __bf16*)p.v + koff,
@@ -43,12 +45,22 @@ __global__ void __launch_bounds__(256, 2) q_sweep_ddo(Params p) {
   // the first streamed tile is requested before the resident operands: the two round trips to memory overlap
   const StreamKeys<MASK> geo(p.mask_off, p.window, p.n_k);
   int j_begin, j_end;  // key tiles this workgroup visits
-  geo.tile_range(q0, WG_ROWS, j_begin, j_end);
+  geo.tile_range(q0, ROWS, j_begin, j_end);
+  // staging: four waves share the rows of a tile; with eight waves each group of four takes two of the four tensors
+  constexpr int NLD = NW == 8 ? NT / 2 : NT;
+  const int half = NW == 8 ? wave >> 2 : 0;
+  const __bf16* srcl[NLD];
+#pragma unroll
+  for (int x = 0; x < NLD; x++) {   // wave-uniform, and the staging instruction wants it in scalar registers
+    const uint64_t a = (uint64_t)(NW == 8 ? (half ? src[NT / 2 + x < NT ? NT / 2 + x : 0] : src[x]) : src[x]);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    srcl[x] = (const __bf16*)(((uint64_t)hi << 32) | lo);
+  }
   Dma<D> dma;
-  dma.init(p.stride_kn, wave, lane);
-  const uint32_t ring_lds = lds_addr(smem);
+  dma.init(p.stride_kn, wave & 3, lane);
+  const uint32_t ring_lds = lds_addr(smem) + half * NLD * TILE;
   const auto stage_tile = [&](int j) {
-    dma.template issue_all<NT>(ring_lds + (j & 1) * STAGE, TILE, src, (int64_t)j * TS * p.stride_kn, wave, p.n_k - j * TS);
+    dma.template issue_all<NLD>(ring_lds + (j & 1) * STAGE, TILE, srcl, (int64_t)j * TS * p.stride_kn, wave & 3, p.n_k - j * TS);
   };
   if (j_begin < j_end) stage_tile(j_begin);
 
@@ -210,10 +222,10 @@ __global__ void __launch_bounds__(256, 2) q_sweep_ddo(Params p) {
 }
 
 template <auto Kernel>
-hipError_t launch(unsigned grid, int smem, hipStream_t s, const Params& p) {
+hipError_t launch(unsigned grid, unsigned threads, int smem, hipStream_t s, const Params& p) {
   const hipError_t e = allow_dynamic_lds<Kernel>(smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(Kernel, dim3(grid), dim3(256), smem, s, p);
+  hipLaunchKernelGGL(Kernel, dim3(grid), dim3(threads), smem, s, p);
   return hipGetLastError();
 }
 
@@ -221,8 +233,15 @@ template <bool F16, int D, int MASK>
 hipError_t launch_ddo_d(const Params& p, int pass, hipStream_t s) {
   const unsigned grid = grid_blocks((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch);
   constexpr int smem = 2 * 4 * TS * 2 * D;
-  if (pass == FHOG_PASS_B_DDO) return launch<q_sweep_ddo<F16, D, MASK, true>>(grid, smem, s, p);
-  return launch<q_sweep_ddo<F16, D, MASK, false>>(grid, smem, s, p);
+  // with plenty of workgroups, 256 queries per workgroup of eight waves (one per CU), as the b sweep does at d = 128
+  const unsigned g8 = grid_blocks((p.n_q + 255) / 256, p.batch);
+  const int w8 = tuning().b8;
+  if (D == 128 && (w8 < 0 ? g8 >= 512 : w8 == 1)) {
+    if (pass == FHOG_PASS_B_DDO) return launch<q_sweep_ddo<F16, D, MASK, true, 8>>(g8, 512, smem, s, p);
+    return launch<q_sweep_ddo<F16, D, MASK, false, 8>>(g8, 512, smem, s, p);
+  }
+  if (pass == FHOG_PASS_B_DDO) return launch<q_sweep_ddo<F16, D, MASK, true>>(grid, 256, smem, s, p);
+  return launch<q_sweep_ddo<F16, D, MASK, false>>(grid, 256, smem, s, p);
 }
 
 }  // namespace

@@ -38,7 +38,7 @@ def pass_of(kernel):
     m = re.match(r"q_sweep_bf16<\w+, \d+, (\d)", kernel)
     if m:
         return int(m.group(1))
-    m = re.match(r"q_sweep_ddo<\w+, \d+, \d, (\w+)>", kernel)
+    m = re.match(r"q_sweep_ddo<\w+, \d+, \d, (\w+)[,>]", kernel)
     if m:
         return 6 if m.group(1) == "true" else 8
     if re.match(r"q_sweep3_pc<\w+, \d+, \d, true>", kernel):
@@ -79,8 +79,8 @@ def compare(w, variants):
     """One table row per (variant, double-backward kernel): average duration, matrix-pipe occupancy, clock, HBM bytes read.
     `variants`: list of (label, directory holding prof_kt, prof_fetch, prof_sq of a run made under that FHOG_TUNE)."""
     P = print
-    P("| FHOG_TUNE | kernel | calls | avg ns | MFMA busy fraction | clock GHz | HBM read MiB | HBM read / algorithmic |")
-    P("|---|---|---|---|---|---|---|---|")
+    P("| FHOG_TUNE | kernel | calls | avg ns | MFMA busy fraction | VALU per MFMA | clock GHz | HBM read MiB | HBM read / algorithmic |")
+    P("|---|---|---|---|---|---|---|---|---|")
     for label, root in variants:
         root = Path(root)
         kt = {short(r["Name"]): r for r in csv.DictReader(open(root / "prof_kt" / "kt_kernel_stats.csv")) if "fhog" in r["Name"]}
@@ -94,7 +94,8 @@ def compare(w, variants):
             d = sq[k]
             cyc, ns = d["SQ_BUSY_CYCLES"] / 32, float(kt[k]["AverageNs"])
             f = fe[k]["FETCH_SIZE"] * sf / 1024
-            P(f"| {label} | {k} | {kt[k]['Calls']} | {ns:.0f} | {d['SQ_VALU_MFMA_BUSY_CYCLES'] / 1024 / cyc:.3f} | {cyc / ns:.2f} | {f:.1f} | "
+            P(f"| {label} | {k} | {kt[k]['Calls']} | {ns:.0f} | {d['SQ_VALU_MFMA_BUSY_CYCLES'] / 1024 / cyc:.3f} | "
+              f"{(d['SQ_INSTS_VALU'] - d['SQ_INSTS_MFMA']) / d['SQ_INSTS_MFMA']:.2f} | {cyc / ns:.2f} | {f:.1f} | "
               f"{f / algorithmic_mib(w, p)[0]:.2f} |")
 
 

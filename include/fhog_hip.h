@@ -106,6 +106,7 @@ extern "C" {
  *   split=0|1         small launches may split their streamed side over several workgroups (needs the workspace of
  *                     fhog_bwdbwd_workspace_hint)
  *   dd64=0|1          dd sweep at d = 128 with 32 | 64 queries per wave
+ *   stage64=0|1       single-role sweeps at d = 64: one | two 32-row tiles staged and consumed per barrier
  * Results do not depend on any of them beyond fp32 summation order (split) - the others are bit-identical. Unknown keys
  * and values are reported on stderr and ignored. */
 typedef struct fhog_bwdbwd_args {
