@@ -402,8 +402,12 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   const int* order = four;
   int first = impl == FHOG_IMPL_BF16 ? 1 : 0, n_pass = 5;
   if (args->schedule == FHOG_SCHEDULE_FUSED_STATS) order = fused, n_pass = 4;
-  if (args->schedule == FHOG_SCHEDULE_DDO_EARLY && impl == FHOG_IMPL_BF16) order = ddo_early, first = 0, n_pass = 4;
-  if (args->schedule == FHOG_SCHEDULE_THREE_SWEEP && impl == FHOG_IMPL_BF16) order = three, first = 0, n_pass = 3;
+  // Passes 6-8 have no split form: a launch too small to fill the GPU whose workspace lets the reference's passes split
+  // their streamed side runs the nearest schedule that can (three sweeps -> fused statistics, ddO early -> four passes).
+  const bool small = granted_split(args, impl, FHOG_PASS_DQ_DDO) > 1;
+  if (args->schedule == FHOG_SCHEDULE_THREE_SWEEP && small) order = fused, n_pass = 4;
+  if (args->schedule == FHOG_SCHEDULE_DDO_EARLY && impl == FHOG_IMPL_BF16 && !small) order = ddo_early, first = 0, n_pass = 4;
+  if (args->schedule == FHOG_SCHEDULE_THREE_SWEEP && impl == FHOG_IMPL_BF16 && !small) order = three, first = 0, n_pass = 3;
   for (int i = first; i < n_pass; i++) {
     const int r = run_pass(args, p, impl, order[i], (hipStream_t)hip_stream);
     if (r != FHOG_OK) return r;

@@ -193,20 +193,29 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_ddo(Params p
       const bf16x4_t do4 = *reinterpret_cast<const bf16x4_t*>(dorow + col);
       bf16x4_t o4 = do4;
       if (!KNOWN_DD) o4 = *reinterpret_cast<const bf16x4_t*>(orow + col);
-      float v[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const float dof = to_f32<F16>(do4[i]);
-        v[i] = acc[cb][4 * g + i];
+        float v = acc[cb][4 * g + i];
         if (!KNOWN_DD) {
           const float of = to_f32<F16>(o4[i]);
           od = __builtin_fmaf(of, dof, od);
-          v[i] = __builtin_fmaf(-dd, of, v[i]);   // (P o ddS) V - dd O = ddP V
+          v = __builtin_fmaf(-dd, of, v);   // (P o ddS) V - dd O = ddP V
         }
-        dot = __builtin_fmaf(dof, v[i], dot);
+        dot = __builtin_fmaf(dof, v, dot);
+        acc[cb][4 * g + i] = v;
       }
-      if (qi < p.n_q) *reinterpret_cast<u32x2_t*>(oddo + col) = pack4<F16>(v[0], v[1], v[2], v[3]);
     }
+  // the stores in a run of their own, so that the eight-byte pieces of a row reach the memory side together
+  if (qi < p.n_q) {
+#pragma unroll
+    for (int cb = 0; cb < NC; cb++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const f32x16_t& y = acc[cb];
+        *reinterpret_cast<u32x2_t*>(oddo + 32 * cb + 8 * g + 4 * h) = pack4<F16>(y[4 * g], y[4 * g + 1], y[4 * g + 2], y[4 * g + 3]);
+      }
+  }
   dot += __shfl_xor(dot, 32);
   if (!KNOWN_DD) {
     od += __shfl_xor(od, 32);

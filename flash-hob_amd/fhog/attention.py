@@ -219,11 +219,12 @@ class AttnBwd(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, q, k, v, o, do, L, scale, causal, window=None):
+    def forward(ctx, q, k, v, o, do, L, scale, causal, window=None, schedule=None):
         ctx.save_for_backward(q, k, v, o, do, L)
         ctx.scale = scale
         ctx.causal = causal
         ctx.window = window
+        ctx.schedule = schedule
         sq = q.shape
         f = (lambda t: t.flatten(0, 1)) if q.dim() == 4 else (lambda t: t)
         dq, dk, dv = attention_backward(f(q), f(k), f(v), f(o), f(do), f(L), scale, causal, window=window)
@@ -234,9 +235,9 @@ class AttnBwd(torch.autograd.Function):
     def backward(ctx, ddq, ddk, ddv):
         q, k, v, o, do, L = ctx.saved_tensors
         dq2, dk2, dv2, ddo = flash_bwdbwd(q, k, v, o, do, ddq.contiguous(), ddk.contiguous(), ddv.contiguous(), L,
-                                          ctx.scale, causal=ctx.causal, window=ctx.window)
+                                          ctx.scale, causal=ctx.causal, window=ctx.window, schedule=ctx.schedule)
         # O and L are caches of (q, k, v): the four results are already total derivatives.
-        return dq2, dk2, dv2, None, ddo, None, None, None, None
+        return dq2, dk2, dv2, None, ddo, None, None, None, None, None
 
 
 class FlashAttention(torch.autograd.Function):
@@ -244,23 +245,25 @@ class FlashAttention(torch.autograd.Function):
     ``FlashAttention2`` (``fhog/triton_flash.py:136-198``), twice differentiable."""
 
     @staticmethod
-    def forward(ctx, q, k, v, is_causal=False, window=None):
+    def forward(ctx, q, k, v, is_causal=False, window=None, schedule=None):
         scale = q.shape[-1] ** -0.5
         o, L = attention_forward(q, k, v, scale, is_causal, window=window)
         ctx.save_for_backward(q, k, v, o, L)
         ctx.is_causal = is_causal
         ctx.window = window
+        ctx.schedule = schedule
         ctx.scale = scale
         return o
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, L = ctx.saved_tensors
-        dq, dk, dv = AttnBwd.apply(q, k, v, o, do.contiguous(), L, ctx.scale, ctx.is_causal, ctx.window)
-        return dq, dk, dv, None, None
+        dq, dk, dv = AttnBwd.apply(q, k, v, o, do.contiguous(), L, ctx.scale, ctx.is_causal, ctx.window, ctx.schedule)
+        return dq, dk, dv, None, None, None
 
 
-def attention(q, k, v, is_causal=False, window: Optional[int] = None):
+def attention(q, k, v, is_causal=False, window: Optional[int] = None, schedule: Optional[str] = None):
     """Twice-differentiable scaled-dot-product attention (scale = d^-1/2). ``is_causal``: False | True |
-    "bottom_right"; ``window``: sliding-window length on top of a causal mask."""
-    return FlashAttention.apply(q, k, v, is_causal, window)
+    "bottom_right"; ``window``: sliding-window length on top of a causal mask; ``schedule``: pass schedule of the
+    double-backward (see :func:`fhog.flash_bwdbwd`; None = the reference's four passes)."""
+    return FlashAttention.apply(q, k, v, is_causal, window, schedule)

@@ -94,8 +94,9 @@ extern "C" {
                                        dK2+dV2. 20 recomputed products. ddP V is formed as (P o ddS) V - dd O with the
                                        caller's 16-bit O: accurate as long as dd_i does not dominate ddS_ij - dd_i.
                                        Schedules 2 and 3 exist in the 16-bit MFMA family; the fp32-MFMA family runs the
-                                       four-pass schedule for them, and launches too small to fill the GPU do not split
-                                       their streamed side in the passes 6, 7 and 8 */
+                                       four-pass schedule for them. Passes 6, 7 and 8 have no split form: a launch too
+                                       small to fill the GPU whose workspace allows a split (ws_bytes) runs the four
+                                       passes (schedule 2) or the fused statistics sweep and passes 3, 4 (schedule 3) */
 
 /* Launch choices (the counterpart of the reference's autotune list, fhog/triton_bwdbwd.py:12-36) are fixed functions of
  * the launch size. For experiments they can be overridden through the environment variable FHOG_TUNE, a comma-separated

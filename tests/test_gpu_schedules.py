@@ -64,6 +64,21 @@ def test_schedules_fp16_and_unit_cotangents(d, schedule):
 
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
+@pytest.mark.parametrize("split", [True, False])
+def test_schedules_on_a_launch_too_small_to_fill_the_gpu(schedule, split):
+    """One head of 4096 tokens is 32 workgroups: with the larger workspace the library runs the nearest schedule whose
+    passes can split their streamed side, with the minimum workspace the schedule itself, unsplit. Same gates either way."""
+    x = with_caches(make_case(1, 4096, 4096, 64, torch.bfloat16, seed=58, grad_std=0.1), 0.125, False)
+    outs = run_fhog(x, 0.125, False, schedule=schedule, split=split, return_stats=True)
+    ref = reference_fp32_gpu(x, 0.125, False)
+    e = errors(outs[:4], ref)
+    assert max(e.values()) < 2e-2, e
+    d, dd, b = outs[4]
+    rowdot = (x["dO"].float() * outs[3].float()).sum(-1)
+    assert normalised_max_error(b, rowdot - d * dd) < 1e-2
+
+
+@pytest.mark.parametrize("schedule", SCHEDULES)
 def test_schedules_against_the_default_one(schedule):
     """Same tensors through the reference schedule and an opt-in one: dK2, dV2 and dQ2 depend on the row statistics
     (dd, b) only, so they move by no more than the statistics' own rounding; ddO is rounded once in both."""
@@ -127,3 +142,25 @@ def test_schedules_full_size_configs(name, heads, schedule):
     e = _full_config(name, 4, schedule, heads=heads)
     print(f"{name} {schedule}: {e}")
     assert max(e.values()) < 2e-2, e
+
+
+@pytest.mark.parametrize("schedule", SCHEDULES)
+def test_schedules_through_the_autograd_chain(schedule):
+    """`fhog.attention(..., schedule=...)`: create_graph=True through FlashAttention -> AttnBwd -> flash_bwdbwd with an
+    opt-in schedule, bf16 tensors, against plain torch attention in fp32 on the same (rounded) tensors."""
+    import fhog
+    g = torch.Generator().manual_seed(57)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).cuda()
+    q, k, v, w = mk(2, 256, 128), mk(2, 256, 128), mk(2, 256, 128), mk(2, 256, 128) * 0.1
+
+    def penalty(attn, cast):
+        qq, kk, vv = (cast(t).clone().requires_grad_(True) for t in (q, k, v))
+        out = attn(qq, kk, vv)
+        gq, gk, gv = torch.autograd.grad((out * cast(w)).sum(), (qq, kk, vv), create_graph=True)
+        loss = gq.float().square().sum() + (gk.float() * gv.float()).sum()
+        return torch.autograd.grad(loss, (qq, kk, vv))
+
+    ours = penalty(lambda a, b, c: fhog.attention(a, b, c, True, schedule=schedule), lambda t: t)
+    ref = penalty(lambda a, b, c: torch.nn.functional.scaled_dot_product_attention(a, b, c, is_causal=True), lambda t: t.float())
+    for a, b in zip(ours, ref):
+        assert normalised_max_error(a, b) < 3e-2   # three bf16 kernels in a row (forward, first backward, double-backward)
