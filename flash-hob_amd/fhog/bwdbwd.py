@@ -151,7 +151,8 @@ def flash_bwdbwd(Q, K, V, O, dO, ddQ, ddK, ddV, L, scale, *, causal=False, windo
             schedules "fused_stats" (22), "ddo_early" (23: four sweeps, the second one yields ``ddO`` together with
             ``b_i = dO_i . ddO_i - d_i dd_i``, the third ``dQ2`` alone) and "three_sweep" (20: ``dd``, ``b`` and ``ddO``
             from one sweep, then ``dQ2``, then ``dK2`` and ``dV2``). The last two exist in the 16-bit kernels; fp32
-            tensors run the reference schedule whatever is asked.
+            tensors run the reference schedule whatever is asked, and a launch too small to fill the GPU (with
+            ``split=True``) runs the nearest schedule whose passes can split their streamed side.
         return_stats: also return the fp32 row vectors ``(d, dd, b)`` of shape like ``L``.
         only_pass: run a single pass (0..5, see fhog._lib.PASS_*) instead of the whole chain; for tests and profiling.
         split: allocate the larger workspace that lets launches too small to fill the GPU split their streamed side over
