@@ -59,7 +59,7 @@ def event_time_ms(fn, iters):
     return event_times_ms(fn, iters)["mean"]
 
 
-def mfma_sustained(dev):
+def mfma_sustained(dev, trips=20000, repeats=2):
     """bf16 MFMA rate of a loop of nothing but MFMAs, on zero and on random operands (TFLOP/s): the rate the chip holds
     under its power limit depends on the operand data; the second figure is the practical ceiling for real tensors."""
     import ctypes
@@ -70,11 +70,15 @@ def mfma_sustained(dev):
     out = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     res = {}
-    for name, mode in (("zeros", 0), ("random", 1)):
+    # the last three: the same random-operand loop with the A operands read from LDS (one 128-bit read per MFMA,
+    # prefetched: the matrix pipe never waits for them), with three VALU instructions per MFMA, and with both - what
+    # the power limit leaves of the MFMA rate for a kernel with the instruction mix of the recomputation sweeps
+    for name, mode in (("zeros", 0), ("random", 1), ("random_lds_read_per_mfma", 2), ("random_lds_read_per_2_mfma", 3),
+                       ("random_3_valu_per_mfma", 4), ("random_lds_read_and_3_valu_per_mfma", 5)):
         flops = ctypes.c_double()
         run = lambda trips: _lib.check(L.fhog_probe_mfma_rate(out.data_ptr(), blocks, trips, mode, ctypes.byref(flops), stream))
-        run(4000)   # warm-up, also lets the clock settle
-        ms = event_time_ms(lambda: run(20000), 2)
+        run(trips)   # warm-up, also lets the clock settle
+        ms = event_time_ms(lambda: run(trips), repeats)
         res[name] = round(flops.value / ms / 1e9, 1)
     return res
 
@@ -184,6 +188,7 @@ def main():
     ap.add_argument("--workload", default=None, help="one of fhog.workloads.WORKLOADS (default: the headline)")
     ap.add_argument("--cpu-heads", type=int, default=32, help="slices of the workload timed on the CPU (0 = skip)")
     ap.add_argument("--profile-only", action="store_true", help="run the timed loop only (for rocprofv3)")
+    ap.add_argument("--probe-only", action="store_true", help="run the MFMA rate probes only and print their figures (for rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU (the path shards over batch*head with no communication); "
@@ -196,6 +201,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a ROCm GPU"
     _lib.lib()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
+    if args.probe_only:
+        print(json.dumps(mfma_sustained(dev, trips=20000, repeats=3)))
+        return
     w = WORKLOADS[args.workload or HEADLINE]
 
     x_cpu = {n: t.flatten(0, 1) for n, t in make_inputs(w, seed=0).items()}
@@ -322,9 +330,15 @@ def main():
     # What a loop of nothing but MFMAs on random operands would leave of the algorithmic figure under the four-pass
     # schedule, which issues 25 products for the 12 it is credited with: the ceiling of `value` on this box.
     sustained = out["mfma_sustained_tflops"]["random"]
+    # ... and the same for a loop that also carries one LDS operand read and three VALU instructions per MFMA, the
+    # instruction mix of the sweeps (still nothing the matrix pipe waits for: profiles/mfma_rate_instruction_mix.md)
+    mix = out["mfma_sustained_tflops"]["random_lds_read_and_3_valu_per_mfma"]
     out["ceiling"] = {"sustained_random_tflops": sustained,
                       "four_pass_algorithmic_tflops": round(sustained * 12 / 25, 1),
-                      "pct_of_ceiling": round(100 * value / (sustained * 12 / 25), 2)}
+                      "pct_of_ceiling": round(100 * value / (sustained * 12 / 25), 2),
+                      "sustained_random_with_sweep_instruction_mix_tflops": mix,
+                      "four_pass_algorithmic_with_mix_tflops": round(mix * 12 / 25, 1),
+                      "pct_of_ceiling_with_mix": round(100 * value / (mix * 12 / 25), 2)}
     if args.cpu_heads > 0:
         out["cpu_baseline"] = cpu_baseline(w, x_cpu, min(args.cpu_heads, w.batch), repeats=2)
     print(json.dumps(out))

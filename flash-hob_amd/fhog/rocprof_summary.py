@@ -99,15 +99,42 @@ def compare(w, variants):
               f"{f / algorithmic_mib(w, p)[0]:.2f} |")
 
 
+PROBE_MODES = {0: "operands all zero", 1: "random operands, nothing but MFMAs",
+               2: "random, one LDS operand read (ds_read_b128) per MFMA", 3: "random, one LDS operand read per two MFMAs",
+               4: "random, three v_fma_f32 per MFMA", 5: "random, one LDS read and three v_fma_f32 per MFMA"}
+
+
+def probe_table(root, trips=20000, blocks=256):
+    """The MFMA rate probes of `bench.py --probe-only`: rate, matrix-pipe occupancy and clock per instruction mix."""
+    root = Path(root)
+    kt = {short(r["Name"]): r for r in csv.DictReader(open(root / "prof_kt" / "kt_kernel_stats.csv")) if "mfma_rate_kernel" in r["Name"]}
+    sq = counters(root / "prof_sq" / "s_counter_collection.csv")
+    flops = blocks * 8.0 * trips * 32 * 32768
+    P = print
+    P("| mode | instruction mix | calls | avg ns | MFMA TFLOP/s | MFMA busy fraction | clock GHz | busy x clock | LDS active fraction |")
+    P("|---|---|---|---|---|---|---|---|---|")
+    for k in sorted(kt):
+        mode = int(re.search(r"<(\d)>", k).group(1))
+        ns, d = float(kt[k]["AverageNs"]), sq[k]
+        cyc = d["SQ_BUSY_CYCLES"] / 32
+        busy = d["SQ_VALU_MFMA_BUSY_CYCLES"] / 1024 / cyc
+        P(f"| {mode} | {PROBE_MODES[mode]} | {kt[k]['Calls']} | {ns:.0f} | {flops / ns / 1e3:.0f} | {busy:.3f} | {cyc / ns:.2f} | "
+          f"{busy * cyc / ns:.2f} | {d['SQ_LDS_IDX_ACTIVE'] / 256 / cyc:.3f} |")
+
+
 def main():
     from fhog.workloads import WORKLOADS
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", required=True)
+    ap.add_argument("--workload", default=None)
+    ap.add_argument("--probe", metavar="DIR", help="instead of a summary: the table of the MFMA rate probes (DIR holds prof_kt and "
+                    "prof_sq of `bench.py --probe-only`)")
     ap.add_argument("--root", default="prof_out", help="directory holding prof_kt, prof_fetch, prof_write, prof_sq")
     ap.add_argument("--note", default="", help="free text appended to the summary")
     ap.add_argument("--compare", nargs="+", metavar="LABEL@DIR", help="instead of a summary: one table over runs made under "
                     "different FHOG_TUNE settings (each DIR holds prof_kt, prof_fetch, prof_sq)")
     args = ap.parse_args()
+    if args.probe:
+        return probe_table(args.probe)
     w = WORKLOADS[args.workload]
     if args.compare:
         return compare(w, [tuple(c.rsplit("@", 1)) for c in args.compare])

@@ -238,11 +238,13 @@ int fhog_attn_fwd(const fhog_attn_args* args, void* hip_stream);
    sweep for dK and dV), without the (batch, n_q, n_k) tensors. */
 int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream);
 
-/* Measurement aid (no counterpart in the reference): enqueue a loop of nothing but bf16 32x32x16 MFMAs on `blocks`
-   workgroups of 8 waves (one per CU fills the chip), `trips` x 32 MFMAs per wave, operands all zero (data_mode 0) or
-   random (data_mode 1). `out`: device buffer of blocks * 512 floats. Returns the FLOPs issued through *flops.
-   Timing it gives the MFMA rate the device sustains at the clock it holds for that operand data, the practical
-   ceiling next to the published peak. */
+/* Measurement aid (no counterpart in the reference): enqueue a loop of bf16 32x32x16 MFMAs on `blocks` workgroups of 8
+   waves (one per CU fills the chip), `trips` x 32 MFMAs per wave. data_mode: 0 operands all zero; 1 random operands in
+   registers (nothing but MFMAs); 2 random, every A operand read from LDS (one 128-bit read per MFMA, prefetched: the
+   matrix pipe never waits); 3 as 2 with one read per two MFMAs; 4 as 1 plus three independent v_fma_f32 per MFMA; 5 one LDS
+   read and three VALU instructions per MFMA, the mix of the recomputation sweeps. `out`: device buffer of blocks * 512
+   floats. Returns the MFMA FLOPs issued through *flops. Timing it gives the MFMA rate the device sustains at the clock it
+   holds for that data and instruction mix, the practical ceiling next to the published peak. */
 int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream);
 
 /* Message for the last failing call on this thread ("" if none). */
