@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: attention double-backward on one MI355X.
 
-One "step" = one call of ``fhog.flash_bwdbwd`` (five launches: d, dd, b, dQ'+ddO, dK'+dV') on
+One "step" = one call of ``fhog.flash_bwdbwd`` (the reference's four passes dd, b, dQ'+ddO, dK'+dV'; the first also writes d) on
 seeded synthetic tensors that are already resident in HBM.  The workload is the configuration the
 metric is quoted on: bf16 causal B=2 H=16 N=4096 d=128.
 

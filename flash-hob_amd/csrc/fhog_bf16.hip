@@ -9,13 +9,14 @@
 // Fused statistics sweep (PASS = 5, opt-in): b_i = sum_j P (E + ddS (dP - d)) - dd_i sum_j P dP
 // needs dd_i only as a factor of a row sum, so dd and b come out of ONE sweep with the five products of pass 2
 // and three running sums per query; the three products of a separate pass 1 are saved.
+// PASS = 7 (opt-in schedules whose second sweep already produced ddO, fhog_bf16_ddo.hip): pass 3 for dQ2 alone, d = 64.
 //
 // The kernels of this file are single-role: a workgroup is 256 threads = 4 wave64 owning 128 stationary rows,
 // two workgroups per CU (the b sweeps at d = 128 also exist with 8 waves and 256 rows, one workgroup per CU, for
 // launches with enough workgroups: half the staging loads per row). Each wave keeps its 32 rows in registers as
 // MFMA B operands (Q, ddQ and, from pass 2 on, dO; K, ddK, V, ddV in pass 4); the other side streams through a
-// two-stage LDS ring of 32-row tiles filled by direct global->LDS loads. First-level products are computed with the streamed rows as M and the stationary
-// rows as N, so every lane owns ONE stationary row: in the Q-tiled sweeps L, d, dd, b are per-lane scalars and a
+// two-stage LDS ring of 32-row tiles filled by direct global->LDS loads. First-level products are computed with the
+// streamed rows as M and the stationary rows as N, so every lane owns ONE stationary row: in the Q-tiled sweeps L, d, dd, b are per-lane scalars and a
 // row sum is a per-lane partial sum, reduced once at the end with a single cross-half shuffle.
 // Passes 3 and 4 at d = 64 fit the second-level products into the same wave (256 registers): the S-shaped
 // accumulators, rounded to 16 bits, are the B operands of those products as they stand (contraction over the
