@@ -180,175 +180,175 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       if (jj + SUB + u < j_end) stage_tile(jj + SUB + u);
 #pragma unroll
     for (int u = 0; u < SUB; u++) {
-    const int j = jj + u;
-    if (SUB > 1 && j >= j_end) continue;
-    const int k0 = j * TS;
-    const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
-    int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
-    if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
-    if (!geo.dead(k0, qw)) {  // else every key of the tile is hidden from this wave
-      const char* stage = smem + (((jj - j_begin) & SUB) + u) * STAGE;
-      // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
-      // is cut into small pieces placed right behind the MFMAs of the same wave, where it runs in the
-      // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
-      //   K  : S += K Q^T, ddS += K ddQ^T
-      //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
-      //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale (fused)
-      //   ddV: E += ddV dO^T           + acc += P (ddS - dd) u   (pass 2: u = dP - d and E' = E - dd d come from
-      //                                  accumulators that start at the row constants; with the tail, acc ends as
-      //                                  sum P (E' + (ddS - dd) u) = sum P (E + ddS u - dP dd))
-      //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
-      //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
-      // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
-      // ddK; w = ddS scale - dd, ddP = P w, z = P (w u - dd d - b) behind ddV; dS' = P E + z in the tail), packs the four
-      // tiles to 16 bits and goes on to the second-level products.
-      constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
-      constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
-      f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
-      if (PASS == 2) {   // u = dP - d and E' = E - kc straight from the matrix pipe (in pass 3 this measured slower)
+      const int j = jj + u;
+      if (SUB > 1 && j >= j_end) continue;
+      const int k0 = j * TS;
+      const bool masked = geo.partial(k0, qw);  // wave-uniform: the block holds hidden keys (mask edge or tensor end)
+      int lo = 0, hi = 0;                       // key k0 + 8g + 4h + e is visible iff lo <= 8g + e <= hi
+      if (masked) keep_branch(), geo.limits(k0, qi, h, lo, hi);
+      if (!geo.dead(k0, qw)) {  // else every key of the tile is hidden from this wave
+        const char* stage = smem + (((jj - j_begin) & SUB) + u) * STAGE;
+        // The products are issued as a stream of NT*KK k-steps (K, then V, ddK, ddV); the elementwise work
+        // is cut into small pieces placed right behind the MFMAs of the same wave, where it runs in the
+        // shadow of the matrix pipe. LDS operands are fetched PF steps ahead.
+        //   K  : S += K Q^T, ddS += K ddQ^T
+        //   V  : dP += V dO^T            + P = exp2(S c - L)                       (pass 2)
+        //   ddK: ddS += ddK Q^T          + P (pass 1) | u = (dP - d) scale (fused)
+        //   ddV: E += ddV dO^T           + acc += P (ddS - dd) u   (pass 2: u = dP - d and E' = E - dd d come from
+        //                                  accumulators that start at the row constants; with the tail, acc ends as
+        //                                  sum P (E' + (ddS - dd) u) = sum P (E + ddS u - dP dd))
+        //                                | acc_dd += P ddS, acc_pdp += P dP, w = ddS u   (fused)
+        //   tail: acc += P ddS (pass 1) | acc += P E (pass 2) | acc += P (w + E) (fused)
+        // Pass 3 (d = 64) runs the same stream with the elementwise work of the producer/consumer kernel (dS = P u behind
+        // ddK; w = ddS scale - dd, ddP = P w, z = P (w u - dd d - b) behind ddV; dS' = P E + z in the tail), packs the four
+        // tiles to 16 bits and goes on to the second-level products.
+        constexpr int kTensorOfPhase[4] = {0, PASS == 1 ? 1 : 2, 1, 3};
+        constexpr int NSTEP = NT * KK, PF = 2, NB = PF + 1, EPK = 16 / KK;
+        f32x16_t s = {0}, dds = {0}, dp = {0}, e = {0}, pv, us, tt;
+        if (PASS == 2) {   // u = dP - d and E' = E - kc straight from the matrix pipe (in pass 3 this measured slower)
 #pragma unroll
-        for (int r = 0; r < 16; r++) dp[r] = -dsum, e[r] = -kc;
-      }
-      uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];   // PASS 3: packed dS, dS', ddP, P (registers 2i, 2i+1)
-      bf16x8_t a[NB];
+          for (int r = 0; r < 16; r++) dp[r] = -dsum, e[r] = -kc;
+        }
+        uint32_t pk_ds[8], pk_ds2[8], pk_ddp[8], pk_p[8];   // PASS 3: packed dS, dS', ddP, P (registers 2i, 2i+1)
+        bf16x8_t a[NB];
 #pragma unroll
-      for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + kTensorOfPhase[i / KK] * TILE, aoff[i % KK]);
+        for (int i = 0; i < PF; i++) a[i] = lds_read128(stage + kTensorOfPhase[i / KK] * TILE, aoff[i % KK]);
 #pragma unroll
-      for (int i = 0; i < NSTEP; i++) {
-        const int ph = (PASS == 1 && i >= KK) ? 2 : i / KK, kk = i % KK, c = i % NB;
-        if (i + PF < NSTEP)
-          a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (ph == 0) {
-          s = mfma<F16>(a[c], Qb[kk], s);
-          dds = mfma<F16>(a[c], ddQb[kk], dds);
-        } else if (ph == 1) {
-          dp = mfma<F16>(a[c], dOb[kk], dp);
+        for (int i = 0; i < NSTEP; i++) {
+          const int ph = (PASS == 1 && i >= KK) ? 2 : i / KK, kk = i % KK, c = i % NB;
+          if (i + PF < NSTEP)
+            a[(i + PF) % NB] = lds_read128(stage + kTensorOfPhase[(i + PF) / KK] * TILE, aoff[(i + PF) % KK]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (ph == 0) {
+            s = mfma<F16>(a[c], Qb[kk], s);
+            dds = mfma<F16>(a[c], ddQb[kk], dds);
+          } else if (ph == 1) {
+            dp = mfma<F16>(a[c], dOb[kk], dp);
 #pragma unroll
-          for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
-        } else if (ph == 2) {
-          dds = mfma<F16>(a[c], Qb[kk], dds);
-          if (P3 && kk == 0 && masked) {
-            keep_branch();
+            for (int r = EPK * kk; r < EPK * (kk + 1); r++) pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+          } else if (ph == 2) {
+            dds = mfma<F16>(a[c], Qb[kk], dds);
+            if (P3 && kk == 0 && masked) {
+              keep_branch();
 #pragma unroll
-            for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
-          }
-#pragma unroll
-          for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
-            if (PASS == 1) {
-              pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
-            } else if (P3) {
-              dp[r] -= dsum;                           // u
-              us[r] = pv[r] * dp[r];                   // dS = P u (scale applied to the accumulator at the end)
-            } else if (PASS == 5) {
-              us[r] = (dp[r] - dsum) * p.scale;
+              for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
             }
-          }
-        } else {
-          e = mfma<F16>(a[c], dOb[kk], e);
-          if (!P3 && kk == 0 && masked) {
-            keep_branch();
 #pragma unroll
-            for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
-          }
-#pragma unroll
-          for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
-            if (PASS == 2) {
-              red = __builtin_fmaf(pv[r] * __builtin_fmaf(dds[r], p.scale, -dd), dp[r], red);   // P w u
-            } else if (P3) {
-              const float w = __builtin_fmaf(dds[r], p.scale, -dd);
-              const float ddp = pv[r] * w;
-              tt[r] = pv[r] * __builtin_fmaf(w, dp[r], -kc);   // z = P (w u - kc)
-              if (r & 1) {
-                if (WITH_DDO) pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
-                pk_ds[r / 2] = pack2<F16>(us[r - 1], us[r]);
-                if (WITH_DDO) pk_p[r / 2] = pack2<F16>(pv[r - 1], pv[r]);
-              } else if (WITH_DDO) {
-                dds[r] = ddp;
+            for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
+              if (PASS == 1) {
+                pv[r] = __builtin_amdgcn_exp2f(s[r] * c_scale_log2 - l_log2);
+              } else if (P3) {
+                dp[r] -= dsum;                           // u
+                us[r] = pv[r] * dp[r];                   // dS = P u (scale applied to the accumulator at the end)
+              } else if (PASS == 5) {
+                us[r] = (dp[r] - dsum) * p.scale;
               }
-            } else {
-              red_dd = __builtin_fmaf(pv[r], dds[r], red_dd);
-              red_pdp = __builtin_fmaf(pv[r], dp[r], red_pdp);
-              us[r] *= dds[r];
+            }
+          } else {
+            e = mfma<F16>(a[c], dOb[kk], e);
+            if (!P3 && kk == 0 && masked) {
+              keep_branch();
+#pragma unroll
+              for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+            }
+#pragma unroll
+            for (int r = EPK * kk; r < EPK * (kk + 1); r++) {
+              if (PASS == 2) {
+                red = __builtin_fmaf(pv[r] * __builtin_fmaf(dds[r], p.scale, -dd), dp[r], red);   // P w u
+              } else if (P3) {
+                const float w = __builtin_fmaf(dds[r], p.scale, -dd);
+                const float ddp = pv[r] * w;
+                tt[r] = pv[r] * __builtin_fmaf(w, dp[r], -kc);   // z = P (w u - kc)
+                if (r & 1) {
+                  if (WITH_DDO) pk_ddp[r / 2] = pack2<F16>(dds[r - 1], ddp);   // dds[r - 1] holds ddP of the even register by now
+                  pk_ds[r / 2] = pack2<F16>(us[r - 1], us[r]);
+                  if (WITH_DDO) pk_p[r / 2] = pack2<F16>(pv[r - 1], pv[r]);
+                } else if (WITH_DDO) {
+                  dds[r] = ddp;
+                }
+              } else {
+                red_dd = __builtin_fmaf(pv[r], dds[r], red_dd);
+                red_pdp = __builtin_fmaf(pv[r], dp[r], red_pdp);
+                us[r] *= dds[r];
+              }
             }
           }
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (PASS == 1) {
-        if (masked) {
-          keep_branch();
+        if (PASS == 1) {
+          if (masked) {
+            keep_branch();
 #pragma unroll
-          for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
-        }
+            for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+          }
 #pragma unroll
-        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], dds[r], red);   // scale applied once at the end
-      } else if (PASS == 2) {
+          for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], dds[r], red);   // scale applied once at the end
+        } else if (PASS == 2) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
-      } else if (P3) {
+          for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], e[r], red);
+        } else if (P3) {
 #pragma unroll
-        for (int r = 0; r < 16; r += 2)
-          pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], tt[r]), __builtin_fmaf(pv[r + 1], e[r + 1], tt[r + 1]));
-        // dQ2^T += ddK^T dS^T + K^T dS'^T ; ddO^T += V^T ddP^T + ddV^T P^T  (stage order K, ddK, V, ddV)
-        constexpr int NIT = 2 * NC;
-        const auto opnd = [](const uint32_t* pk, int t) {
-          return __builtin_bit_cast(bf16x8_t, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]});
-        };
-        constexpr int NX = WITH_DDO ? 4 : 2;   // staged tensors the second level reads: K, ddK (, V, ddV)
-        bf16x8_t ta[2][NX];
+          for (int r = 0; r < 16; r += 2)
+            pk_ds2[r / 2] = pack2<F16>(__builtin_fmaf(pv[r], e[r], tt[r]), __builtin_fmaf(pv[r + 1], e[r + 1], tt[r + 1]));
+          // dQ2^T += ddK^T dS^T + K^T dS'^T ; ddO^T += V^T ddP^T + ddV^T P^T  (stage order K, ddK, V, ddV)
+          constexpr int NIT = 2 * NC;
+          const auto opnd = [](const uint32_t* pk, int t) {
+            return __builtin_bit_cast(bf16x8_t, u32x4_t{pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]});
+          };
+          constexpr int NX = WITH_DDO ? 4 : 2;   // staged tensors the second level reads: K, ddK (, V, ddV)
+          bf16x8_t ta[2][NX];
 #pragma unroll
-        for (int x = 0; x < NX; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
-        if (WITH_DDO) {
+          for (int x = 0; x < NX; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+          if (WITH_DDO) {
 #pragma unroll
-          for (int it = 0; it < NIT; it++) {
-            const int t = it / NC, cb = it % NC, c = it & 1;
-            if (it + 1 < NIT) {
-              const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+            for (int it = 0; it < NIT; it++) {
+              const int t = it / NC, cb = it % NC, c = it & 1;
+              if (it + 1 < NIT) {
+                const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
 #pragma unroll
-              for (int x = 0; x < NX; x++)
-                ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+                for (int x = 0; x < NX; x++)
+                  ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+              acc_dq[cb] = mfma<F16>(ta[c][1], opnd(pk_ds, t), acc_dq[cb]);
+              acc_ddo[cb] = mfma<F16>(ta[c][NX - 2], opnd(pk_ddp, t), acc_ddo[cb]);
+              acc_dq[cb] = mfma<F16>(ta[c][0], opnd(pk_ds2, t), acc_dq[cb]);
+              acc_ddo[cb] = mfma<F16>(ta[c][NX - 1], opnd(pk_p, t), acc_ddo[cb]);
+              __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            acc_dq[cb] = mfma<F16>(ta[c][1], opnd(pk_ds, t), acc_dq[cb]);
-            acc_ddo[cb] = mfma<F16>(ta[c][NX - 2], opnd(pk_ddp, t), acc_ddo[cb]);
-            acc_dq[cb] = mfma<F16>(ta[c][0], opnd(pk_ds2, t), acc_dq[cb]);
-            acc_ddo[cb] = mfma<F16>(ta[c][NX - 1], opnd(pk_p, t), acc_ddo[cb]);
-            __builtin_amdgcn_sched_barrier(0);
+          } else {
+            // dQ2 alone: two column blocks per round, so that the MFMAs on one accumulator are two instructions apart
+            constexpr int NP = NC / 2;
+            bf16x8_t tb[2][2][2];   // [buffer][column block of the pair][K | ddK]
+            const auto read_tb = [&](int buf, int it) {
+              const int t1 = it / NP, cp1 = it % NP;
+#pragma unroll
+              for (int cl = 0; cl < 2; cl++)
+#pragma unroll
+                for (int x = 0; x < 2; x++)
+                  tb[buf][cl][x] = lds_read_tr_pre(stage + troff[2 * cp1 + cl][0], stage + troff[2 * cp1 + cl][1], x * TILE + t1 * 16 * 2 * D);
+            };
+#pragma unroll
+            for (int x = 0; x < 2; x++) tb[0][0][x] = ta[0][x];
+#pragma unroll
+            for (int x = 0; x < 2; x++) tb[0][1][x] = lds_read_tr_pre(stage + troff[1][0], stage + troff[1][1], x * TILE);
+#pragma unroll
+            for (int it = 0; it < 2 * NP; it++) {
+              const int t = it / NP, cp = it % NP, c = it & 1;
+              if (it + 1 < 2 * NP) read_tb(c ^ 1, it + 1);
+              __builtin_amdgcn_sched_barrier(0);
+              acc_dq[2 * cp] = mfma<F16>(tb[c][0][1], opnd(pk_ds, t), acc_dq[2 * cp]);
+              acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][1], opnd(pk_ds, t), acc_dq[2 * cp + 1]);
+              acc_dq[2 * cp] = mfma<F16>(tb[c][0][0], opnd(pk_ds2, t), acc_dq[2 * cp]);
+              acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][0], opnd(pk_ds2, t), acc_dq[2 * cp + 1]);
+              __builtin_amdgcn_sched_barrier(0);
+            }
           }
         } else {
-          // dQ2 alone: two column blocks per round, so that the MFMAs on one accumulator are two instructions apart
-          constexpr int NP = NC / 2;
-          bf16x8_t tb[2][2][2];   // [buffer][column block of the pair][K | ddK]
-          const auto read_tb = [&](int buf, int it) {
-            const int t1 = it / NP, cp1 = it % NP;
 #pragma unroll
-            for (int cl = 0; cl < 2; cl++)
-#pragma unroll
-              for (int x = 0; x < 2; x++)
-                tb[buf][cl][x] = lds_read_tr_pre(stage + troff[2 * cp1 + cl][0], stage + troff[2 * cp1 + cl][1], x * TILE + t1 * 16 * 2 * D);
-          };
-#pragma unroll
-          for (int x = 0; x < 2; x++) tb[0][0][x] = ta[0][x];
-#pragma unroll
-          for (int x = 0; x < 2; x++) tb[0][1][x] = lds_read_tr_pre(stage + troff[1][0], stage + troff[1][1], x * TILE);
-#pragma unroll
-          for (int it = 0; it < 2 * NP; it++) {
-            const int t = it / NP, cp = it % NP, c = it & 1;
-            if (it + 1 < 2 * NP) read_tb(c ^ 1, it + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            acc_dq[2 * cp] = mfma<F16>(tb[c][0][1], opnd(pk_ds, t), acc_dq[2 * cp]);
-            acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][1], opnd(pk_ds, t), acc_dq[2 * cp + 1]);
-            acc_dq[2 * cp] = mfma<F16>(tb[c][0][0], opnd(pk_ds2, t), acc_dq[2 * cp]);
-            acc_dq[2 * cp + 1] = mfma<F16>(tb[c][1][0], opnd(pk_ds2, t), acc_dq[2 * cp + 1]);
-            __builtin_amdgcn_sched_barrier(0);
-          }
+          for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], us[r] + e[r], red);
         }
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; r++) red = __builtin_fmaf(pv[r], us[r] + e[r], red);
       }
-    }
     }
     dma_wait();
     __syncthreads();
@@ -667,93 +667,93 @@ __global__ void __launch_bounds__(256, 2) k_sweep_bf16(Params p) {
       }
 #pragma unroll
     for (int u = 0; u < SUB; u++) {
-    const int j = jj + u;
-    if (SUB > 1 && j >= t_end) continue;
-    const int qb = j * TS;
-    if (!geo.dead(qb, kw)) {  // else no query of the tile sees a key of this wave
-      const char* stage = smem + (grp + u) * STAGE;
-      const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
-      // five first-level products in one stream of KK k-steps; the three staged operands of step kk + 1 are
-      // fetched before the MFMAs of step kk: S = Q K^T, ddS = ddQ K^T + Q ddK^T, dP = dO V^T, E = dO ddV^T
-      // register 4g + i belongs to query qb + 8g + 4h + i: its statistics come from the staged arrays. The accumulators
-      // of dP and E start at -d and -(dd d + b): u = dP - d and E' = E - dd d - b come straight from the matrix pipe.
-      f32x16_t s = {0}, dds = {0}, dp, e;
+      const int j = jj + u;
+      if (SUB > 1 && j >= t_end) continue;
+      const int qb = j * TS;
+      if (!geo.dead(qb, kw)) {  // else no query of the tile sees a key of this wave
+        const char* stage = smem + (grp + u) * STAGE;
+        const float* stat = reinterpret_cast<const float*>(stage + 3 * TILE);
+        // five first-level products in one stream of KK k-steps; the three staged operands of step kk + 1 are
+        // fetched before the MFMAs of step kk: S = Q K^T, ddS = ddQ K^T + Q ddK^T, dP = dO V^T, E = dO ddV^T
+        // register 4g + i belongs to query qb + 8g + 4h + i: its statistics come from the staged arrays. The accumulators
+        // of dP and E start at -d and -(dd d + b): u = dP - d and E' = E - dd d - b come straight from the matrix pipe.
+        f32x16_t s = {0}, dds = {0}, dp, e;
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const f32x4_t md4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
-        const f32x4_t mk4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
+        for (int g = 0; g < 4; g++) {
+          const f32x4_t md4 = *reinterpret_cast<const f32x4_t*>(stat + 1 * TS + 8 * g + 4 * h);
+          const f32x4_t mk4 = *reinterpret_cast<const f32x4_t*>(stat + 3 * TS + 8 * g + 4 * h);
 #pragma unroll
-        for (int i = 0; i < 4; i++) dp[4 * g + i] = md4[i], e[4 * g + i] = mk4[i];
-      }
-      bf16x8_t a[2][3];
-#pragma unroll
-      for (int x = 0; x < 3; x++) a[0][x] = lds_read128(stage + x * TILE, aoff[0]);
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++) {
-        const int c = kk & 1;
-        if (kk + 1 < KK) {
-#pragma unroll
-          for (int x = 0; x < 3; x++) a[c ^ 1][x] = lds_read128(stage + x * TILE, aoff[kk + 1]);
+          for (int i = 0; i < 4; i++) dp[4 * g + i] = md4[i], e[4 * g + i] = mk4[i];
         }
-        __builtin_amdgcn_sched_barrier(0);
-        s = mfma<F16>(a[c][0], Kb[kk], s);
-        dds = mfma<F16>(a[c][1], Kb[kk], dds);
-        dp = mfma<F16>(a[c][2], Vb[kk], dp);
-        dds = mfma<F16>(a[c][0], ddKb[kk], dds);
-        e = mfma<F16>(a[c][2], ddVb[kk], e);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      f32x16_t pv;
+        bf16x8_t a[2][3];
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 0 * TS + 8 * g + 4 * h);
+        for (int x = 0; x < 3; x++) a[0][x] = lds_read128(stage + x * TILE, aoff[0]);
 #pragma unroll
-        for (int i = 0; i < 4; i++) pv[4 * g + i] = __builtin_amdgcn_exp2f(s[4 * g + i] * c_scale_log2 - l4[i]);
-      }
-      if (geo.partial(qb, kw)) {  // wave-uniform: the block holds hidden (query, key) pairs (mask edge or tensor end)
-        int lo, hi;                // query row 8g + 4h + i of the tile counts iff lo <= 8g + i <= hi
-        geo.limits(qb, kj, h, lo, hi);
-        keep_branch();
+        for (int kk = 0; kk < KK; kk++) {
+          const int c = kk & 1;
+          if (kk + 1 < KK) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
-      }
-      // dS -> s, dS' -> e, ddP -> dds (in place; scale on dS, dS' is applied to the accumulators at the end)
+            for (int x = 0; x < 3; x++) a[c ^ 1][x] = lds_read128(stage + x * TILE, aoff[kk + 1]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          s = mfma<F16>(a[c][0], Kb[kk], s);
+          dds = mfma<F16>(a[c][1], Kb[kk], dds);
+          dp = mfma<F16>(a[c][2], Vb[kk], dp);
+          dds = mfma<F16>(a[c][0], ddKb[kk], dds);
+          e = mfma<F16>(a[c][2], ddVb[kk], e);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        f32x16_t pv;
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
+        for (int g = 0; g < 4; g++) {
+          const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(stat + 0 * TS + 8 * g + 4 * h);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int r = 4 * g + i;
-          const float pr = pv[r];
-          dds[r] = pr * __builtin_fmaf(dds[r], p.scale, -dd4[i]);   // ddP = P (ddS - dd)
-          s[r] = pr * dp[r];                                         // dS = P u
-          e[r] = __builtin_fmaf(pr, e[r], dds[r] * dp[r]);           // dS' = P (E' + (ddS - dd) u)
+          for (int i = 0; i < 4; i++) pv[4 * g + i] = __builtin_amdgcn_exp2f(s[4 * g + i] * c_scale_log2 - l4[i]);
+        }
+        if (geo.partial(qb, kw)) {  // wave-uniform: the block holds hidden (query, key) pairs (mask edge or tensor end)
+          int lo, hi;                // query row 8g + 4h + i of the tile counts iff lo <= 8g + i <= hi
+          geo.limits(qb, kj, h, lo, hi);
+          keep_branch();
+#pragma unroll
+          for (int r = 0; r < 16; r++) pv[r] = in_limits(r, lo, hi) ? pv[r] : 0.f;
+        }
+        // dS -> s, dS' -> e, ddP -> dds (in place; scale on dS, dS' is applied to the accumulators at the end)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const f32x4_t dd4 = *reinterpret_cast<const f32x4_t*>(stat + 2 * TS + 8 * g + 4 * h);
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int r = 4 * g + i;
+            const float pr = pv[r];
+            dds[r] = pr * __builtin_fmaf(dds[r], p.scale, -dd4[i]);   // ddP = P (ddS - dd)
+            s[r] = pr * dp[r];                                         // dS = P u
+            e[r] = __builtin_fmaf(pr, e[r], dds[r] * dp[r]);           // dS' = P (E' + (ddS - dd) u)
+          }
+        }
+        const bf16x8_t op_ds[2] = {pack_operand<F16>(s, 0), pack_operand<F16>(s, 1)};
+        const bf16x8_t op_ds2[2] = {pack_operand<F16>(e, 0), pack_operand<F16>(e, 1)};
+        const bf16x8_t op_ddp[2] = {pack_operand<F16>(dds, 0), pack_operand<F16>(dds, 1)};
+        // dK2^T += ddQ^T dS + Q^T dS' ; dV2^T += dO^T ddP   (stage order Q, ddQ, dO)
+        constexpr int NIT = 2 * NC;
+        bf16x8_t ta[2][3];
+#pragma unroll
+        for (int x = 0; x < 3; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+          const int t = it / NC, cb = it % NC, c = it & 1;
+          if (it + 1 < NIT) {
+            const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
+#pragma unroll
+            for (int x = 0; x < 3; x++)
+              ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          acc_dk[cb] = mfma<F16>(ta[c][1], op_ds[t], acc_dk[cb]);
+          acc_dv[cb] = mfma<F16>(ta[c][2], op_ddp[t], acc_dv[cb]);
+          acc_dk[cb] = mfma<F16>(ta[c][0], op_ds2[t], acc_dk[cb]);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
-      const bf16x8_t op_ds[2] = {pack_operand<F16>(s, 0), pack_operand<F16>(s, 1)};
-      const bf16x8_t op_ds2[2] = {pack_operand<F16>(e, 0), pack_operand<F16>(e, 1)};
-      const bf16x8_t op_ddp[2] = {pack_operand<F16>(dds, 0), pack_operand<F16>(dds, 1)};
-      // dK2^T += ddQ^T dS + Q^T dS' ; dV2^T += dO^T ddP   (stage order Q, ddQ, dO)
-      constexpr int NIT = 2 * NC;
-      bf16x8_t ta[2][3];
-#pragma unroll
-      for (int x = 0; x < 3; x++) ta[0][x] = lds_read_tr_pre(stage + troff[0][0], stage + troff[0][1], x * TILE);
-#pragma unroll
-      for (int it = 0; it < NIT; it++) {
-        const int t = it / NC, cb = it % NC, c = it & 1;
-        if (it + 1 < NIT) {
-          const int t1 = (it + 1) / NC, cb1 = (it + 1) % NC;
-#pragma unroll
-          for (int x = 0; x < 3; x++)
-            ta[c ^ 1][x] = lds_read_tr_pre(stage + troff[cb1][0], stage + troff[cb1][1], x * TILE + t1 * 16 * 2 * D);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        acc_dk[cb] = mfma<F16>(ta[c][1], op_ds[t], acc_dk[cb]);
-        acc_dv[cb] = mfma<F16>(ta[c][2], op_ddp[t], acc_dv[cb]);
-        acc_dk[cb] = mfma<F16>(ta[c][0], op_ds2[t], acc_dk[cb]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
     }
     if (jj + SUB < t_end) {
       wait_vm0();
