@@ -73,8 +73,12 @@ def mfma_sustained(dev, trips=20000, repeats=2):
     # the last three: the same random-operand loop with the A operands read from LDS (one 128-bit read per MFMA,
     # prefetched: the matrix pipe never waits for them), with three VALU instructions per MFMA, and with both - what
     # the power limit leaves of the MFMA rate for a kernel with the instruction mix of the recomputation sweeps
+    # the last: modes 1, 2, 4 with ONE wave per SIMD, where a wave's LDS reads and VALU instructions have only its own MFMAs
+    # to hide behind: what they cost a wave in issue time (the figures above are what they cost in clock)
     for name, mode in (("zeros", 0), ("random", 1), ("random_lds_read_per_mfma", 2), ("random_lds_read_per_2_mfma", 3),
-                       ("random_3_valu_per_mfma", 4), ("random_lds_read_and_3_valu_per_mfma", 5)):
+                       ("random_3_valu_per_mfma", 4), ("random_lds_read_and_3_valu_per_mfma", 5),
+                       ("one_wave_per_simd_random", 9), ("one_wave_per_simd_lds_read_per_mfma", 10),
+                       ("one_wave_per_simd_3_valu_per_mfma", 12), ("one_wave_per_simd_lds_read_and_3_valu_per_mfma", 13)):
         flops = ctypes.c_double()
         run = lambda trips: _lib.check(L.fhog_probe_mfma_rate(out.data_ptr(), blocks, trips, mode, ctypes.byref(flops), stream))
         run(trips)   # warm-up, also lets the clock settle

@@ -437,11 +437,12 @@ size_t fhog_static_ws_bytes(void) { return (size_t)FHOG_STATIC_WS_BYTES; }
 
 int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream) {
   if (!out || !flops) return fail(FHOG_E_NULL, "out or flops is NULL");
-  if (blocks < 1 || blocks > 65535 || trips < 1 || data_mode < 0 || data_mode > 5)
-    return fail(FHOG_E_SHAPE, "blocks in 1..65535, trips >= 1, data_mode 0..5");
-  const hipError_t e = fhog::launch_mfma_rate(out, blocks, trips, data_mode, (hipStream_t)hip_stream);
+  const int mix = data_mode & 7, waves = (data_mode & 8) ? 4 : 8;
+  if (blocks < 1 || blocks > 65535 || trips < 1 || data_mode < 0 || data_mode > 13 || mix > 5)
+    return fail(FHOG_E_SHAPE, "blocks in 1..65535, trips >= 1, data_mode 0..5 or 8..13");
+  const hipError_t e = fhog::launch_mfma_rate(out, blocks, trips, mix, waves, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(FHOG_E_LAUNCH, "MFMA rate probe: HIP error %d (%s)", (int)e, hipGetErrorString(e));
-  *flops = (double)blocks * 8.0 * trips * 32.0 * 32768.0;
+  *flops = (double)blocks * waves * trips * 32.0 * 32768.0;
   return FHOG_OK;
 }
 

@@ -112,7 +112,7 @@ hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s);          
 hipError_t launch_attn_bf16(const AttnParams& p, int which, hipStream_t s);         // 0 forward, 1 dQ, 2 dK and dV
 hipError_t launch_attn_fp32(const AttnParams& p, int dtype, int which, hipStream_t s);  // same, fp32 MFMA (fp32 tensors, d = 32)
 hipError_t launch_attn_bwd_k_pc(const AttnParams& p, hipStream_t s);                // dK and dV at d = 128 (producer/consumer)
-hipError_t launch_mfma_rate(float* out, int blocks, int trips, int data_mode, hipStream_t s);  // measurement aid
+hipError_t launch_mfma_rate(float* out, int blocks, int trips, int data_mode, int waves, hipStream_t s);  // measurement aid
 bool bf16_shape_supported(int64_t n_q, int64_t n_k, int64_t d, int causal);
 
 }  // namespace fhog

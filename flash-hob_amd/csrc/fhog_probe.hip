@@ -17,14 +17,15 @@ __device__ __forceinline__ uint32_t xorshift(uint32_t& s) {
   return s;
 }
 
-// 8 waves per CU (two per SIMD), four independent accumulators per wave, 32 MFMAs per loop trip.
+// 8 waves per CU (two per SIMD; launched with 256 threads: four waves, one per SIMD, and every instruction of a wave then
+// has only that wave's own MFMAs to hide behind), four independent accumulators per wave, 32 MFMAs per loop trip.
 // MODE 0: all operands zero; 1: random values in (-2, 2), operands in registers;
 //      2: as 1, every MFMA takes its A operand from LDS (one ds_read_b128 per MFMA, fetched one group of four ahead);
 //      3: as 2 with every operand read feeding two MFMAs (the ratio of a wave that keeps 64 stationary rows);
 //      4: as 1 plus three independent v_fma_f32 per MFMA;
 //      5: 2 and 4 together (one LDS read and three VALU instructions per MFMA: the mix of the recomputation sweeps).
-template <int MODE>
-__global__ void __launch_bounds__(512) mfma_rate_kernel(float* out, int trips) {
+template <int MODE, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) mfma_rate_kernel(float* out, int trips) {
   constexpr bool RANDOM = MODE != 0, LDS = MODE == 2 || MODE == 3 || MODE == 5, VALU = MODE == 4 || MODE == 5;
   constexpr int LDS_BYTES = 32 * 1024;
   __shared__ __attribute__((aligned(16))) char pool[LDS ? LDS_BYTES : 16];
@@ -39,7 +40,7 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(float* out, int trips) {
       b[i][e] = (__bf16)vb;
     }
   if (LDS) {   // 32 KiB of random bf16 values in (-2, 2): 32 tiles of 1 KiB, one per operand read
-    for (int o = l * 16; o < LDS_BYTES; o += 512 * 16) {
+    for (int o = l * 16; o < LDS_BYTES; o += 64 * WAVES * 16) {
       bf16x8_t v;
       for (int e = 0; e < 8; e++) v[e] = (__bf16)(((int)(xorshift(st) & 0xffff) - 32768) / 16384.0f);
       *reinterpret_cast<bf16x8_t*>(pool + o) = v;
@@ -94,19 +95,21 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(float* out, int trips) {
 
 }  // namespace
 
-// Launches the loop on `blocks` workgroups of 512 threads; `out` needs blocks * 512 floats. FLOPs issued:
-// blocks * 8 waves * trips * 32 MFMAs * 32768.
-hipError_t launch_mfma_rate(float* out, int blocks, int trips, int data_mode, hipStream_t s) {
-  const dim3 grid((unsigned)blocks), block(512);
+// Launches the loop on `blocks` workgroups of `waves` (4 or 8) waves; `out` needs blocks * 512 floats. FLOPs issued:
+// blocks * waves * trips * 32 MFMAs * 32768.
+hipError_t launch_mfma_rate(float* out, int blocks, int trips, int data_mode, int waves, hipStream_t s) {
+  const dim3 grid((unsigned)blocks), block(64u * (unsigned)waves);
+#define FHOG_PROBE(M)                                                                                  \
+  case M:                                                                                              \
+    if (waves == 8) hipLaunchKernelGGL((mfma_rate_kernel<M, 8>), grid, block, 0, s, out, trips);       \
+    else hipLaunchKernelGGL((mfma_rate_kernel<M, 4>), grid, block, 0, s, out, trips);                  \
+    break;
+  if (waves != 4 && waves != 8) return hipErrorInvalidValue;
   switch (data_mode) {
-    case 0: hipLaunchKernelGGL(mfma_rate_kernel<0>, grid, block, 0, s, out, trips); break;
-    case 1: hipLaunchKernelGGL(mfma_rate_kernel<1>, grid, block, 0, s, out, trips); break;
-    case 2: hipLaunchKernelGGL(mfma_rate_kernel<2>, grid, block, 0, s, out, trips); break;
-    case 3: hipLaunchKernelGGL(mfma_rate_kernel<3>, grid, block, 0, s, out, trips); break;
-    case 4: hipLaunchKernelGGL(mfma_rate_kernel<4>, grid, block, 0, s, out, trips); break;
-    case 5: hipLaunchKernelGGL(mfma_rate_kernel<5>, grid, block, 0, s, out, trips); break;
+    FHOG_PROBE(0) FHOG_PROBE(1) FHOG_PROBE(2) FHOG_PROBE(3) FHOG_PROBE(4) FHOG_PROBE(5)
     default: return hipErrorInvalidValue;
   }
+#undef FHOG_PROBE
   return hipGetLastError();
 }
 

@@ -105,21 +105,26 @@ PROBE_MODES = {0: "operands all zero", 1: "random operands, nothing but MFMAs",
 
 
 def probe_table(root, trips=20000, blocks=256):
-    """The MFMA rate probes of `bench.py --probe-only`: rate, matrix-pipe occupancy and clock per instruction mix."""
+    """The MFMA rate probes of `bench.py --probe-only`: rate, matrix-pipe occupancy and clock per instruction mix and
+    number of waves per SIMD (kernel `mfma_rate_kernel<mode, waves per workgroup>`)."""
     root = Path(root)
     kt = {short(r["Name"]): r for r in csv.DictReader(open(root / "prof_kt" / "kt_kernel_stats.csv")) if "mfma_rate_kernel" in r["Name"]}
     sq = counters(root / "prof_sq" / "s_counter_collection.csv")
-    flops = blocks * 8.0 * trips * 32 * 32768
     P = print
-    P("| mode | instruction mix | calls | avg ns | MFMA TFLOP/s | MFMA busy fraction | clock GHz | busy x clock | LDS active fraction |")
-    P("|---|---|---|---|---|---|---|---|---|")
-    for k in sorted(kt):
-        mode = int(re.search(r"<(\d)>", k).group(1))
-        ns, d = float(kt[k]["AverageNs"]), sq[k]
-        cyc = d["SQ_BUSY_CYCLES"] / 32
-        busy = d["SQ_VALU_MFMA_BUSY_CYCLES"] / 1024 / cyc
-        P(f"| {mode} | {PROBE_MODES[mode]} | {kt[k]['Calls']} | {ns:.0f} | {flops / ns / 1e3:.0f} | {busy:.3f} | {cyc / ns:.2f} | "
-          f"{busy * cyc / ns:.2f} | {d['SQ_LDS_IDX_ACTIVE'] / 256 / cyc:.3f} |")
+    P("| mode | waves per SIMD | instruction mix | calls | avg ns | MFMA TFLOP/s | MFMA busy fraction | clock GHz | busy x clock | "
+      "cycles per MFMA and wave | LDS active fraction |")
+    P("|---|---|---|---|---|---|---|---|---|---|---|")
+    for waves in (8, 4):
+        for mode in sorted(PROBE_MODES):
+            k = f"mfma_rate_kernel<{mode}, {waves}>(float*, int)"
+            if k not in kt or k not in sq:
+                continue
+            flops = blocks * float(waves) * trips * 32 * 32768
+            ns, d = float(kt[k]["AverageNs"]), sq[k]
+            cyc = d["SQ_BUSY_CYCLES"] / 32
+            busy = d["SQ_VALU_MFMA_BUSY_CYCLES"] / 1024 / cyc
+            P(f"| {mode + (8 if waves == 4 else 0)} | {waves // 4} | {PROBE_MODES[mode]} | {kt[k]['Calls']} | {ns:.0f} | {flops / ns / 1e3:.0f} | "
+              f"{busy:.3f} | {cyc / ns:.2f} | {busy * cyc / ns:.2f} | {cyc / (trips * 32):.1f} | {d['SQ_LDS_IDX_ACTIVE'] / 256 / cyc:.3f} |")
 
 
 def main():

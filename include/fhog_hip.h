@@ -242,8 +242,9 @@ int fhog_attn_bwd(const fhog_attn_args* args, void* hip_stream);
    waves (one per CU fills the chip), `trips` x 32 MFMAs per wave. data_mode: 0 operands all zero; 1 random operands in
    registers (nothing but MFMAs); 2 random, every A operand read from LDS (one 128-bit read per MFMA, prefetched: the
    matrix pipe never waits); 3 as 2 with one read per two MFMAs; 4 as 1 plus three independent v_fma_f32 per MFMA; 5 one LDS
-   read and three VALU instructions per MFMA, the mix of the recomputation sweeps. `out`: device buffer of blocks * 512
-   floats. Returns the MFMA FLOPs issued through *flops. Timing it gives the MFMA rate the device sustains at the clock it
+   read and three VALU instructions per MFMA, the mix of the recomputation sweeps; data_mode + 8 (8..13): the same loops on
+   workgroups of 4 waves, one wave per SIMD, where nothing but a wave's own MFMAs can hide its other instructions. `out`:
+   device buffer of blocks * 512 floats. Returns the MFMA FLOPs issued through *flops. Timing it gives the MFMA rate the device sustains at the clock it
    holds for that data and instruction mix, the practical ceiling next to the published peak. */
 int fhog_probe_mfma_rate(float* out, int blocks, int trips, int data_mode, double* flops, void* hip_stream);
 

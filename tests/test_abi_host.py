@@ -198,7 +198,8 @@ def test_probe_rejects_bad_arguments(L):
     flops = ctypes.c_double()
     assert L.fhog_probe_mfma_rate(None, 256, 10, 0, ctypes.byref(flops), None) == -1
     assert L.fhog_probe_mfma_rate(0x10000, 0, 10, 0, ctypes.byref(flops), None) == -2
-    assert L.fhog_probe_mfma_rate(0x10000, 256, 10, 6, ctypes.byref(flops), None) == -2
+    for mode in (6, 7, 14, 15, 16):
+        assert L.fhog_probe_mfma_rate(0x10000, 256, 10, mode, ctypes.byref(flops), None) == -2
     assert L.fhog_probe_mfma_rate(0x10000, 256, 10, -1, ctypes.byref(flops), None) == -2
 
 

@@ -689,14 +689,17 @@ def test_mfma_rate_probe_runs():
     L = _lib.lib()
     out = torch.full((8 * 512,), float("nan"), device="cuda:0")
     flops = ctypes.c_double()
-    for mode in range(6):   # zeros; random; random with LDS operand reads and / or VALU side work in the stream
+    # zeros; random; random with LDS operand reads and / or VALU side work in the stream; + 8: one wave per SIMD
+    for mode in list(range(6)) + list(range(8, 14)):
+        waves = 4 if mode & 8 else 8
         out.fill_(float("nan"))
         _lib.check(L.fhog_probe_mfma_rate(out.data_ptr(), 8, 100, mode, ctypes.byref(flops),
                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
         torch.cuda.synchronize()
-        assert flops.value == 8 * 8 * 100 * 32 * 32768
-        assert torch.isfinite(out).all()
-        assert mode == 0 or out.abs().max() > 1e-20   # random operands leave non-zero sums
+        assert flops.value == 8 * waves * 100 * 32 * 32768
+        written = out.view(8, 512)[:, :64 * waves]
+        assert torch.isfinite(written).all()
+        assert mode & 7 == 0 or written.abs().max() > 1e-20   # random operands leave non-zero sums
 
 
 def test_autograd_chain_with_a_sliding_window():
