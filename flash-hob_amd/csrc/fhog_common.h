@@ -59,7 +59,7 @@ struct Params {
 //   b8=0|1             b / dd+b sweeps at d = 128: 128-row workgroups of 4 waves | 256-row workgroups of 8 waves
 //                      (default: 8 waves when that still gives 512 workgroups)
 //   order=slice|tile   workgroup order within an XCD (default: tile-major with a mask, slice after slice without)
-//   split=0|1          let small launches split their streamed side (default 0: measured equal within 1 %)
+//   split=0|1          let launches too small to fill the GPU split their streamed side over several workgroups (default 1)
 //   dd64=0|1           dd sweep at d = 128: 32 | 64 queries per wave (default: 64 when that still gives 2048 workgroups)
 //   stage64=0|1        single-role sweeps at d = 64: one | two 32-row tiles staged and consumed per barrier (default 0: measured equal within 1 %)
 struct Tuning {
