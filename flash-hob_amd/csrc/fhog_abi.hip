@@ -247,6 +247,10 @@ fhog::AttnParams to_attn_params(const fhog_attn_args* a) {
   p.causal = a->causal != FHOG_MASK_NONE;
   p.f16 = a->dtype == FHOG_DTYPE_FP16;
   mask_params(a->causal, a->window, a->n_q, a->n_k, &p.mask_off, &p.window);
+  // as in run_pass: tile-major with a mask, until a slice alone has tiles enough to balance the end of a launch
+  const int order = fhog::tuning().order;
+  p.tile_major_q = order < 0 ? (p.causal && a->n_q < 16384) : order;
+  p.tile_major_k = order < 0 ? (p.causal && a->n_k < 16384) : order;
   return p;
 }
 

@@ -68,6 +68,7 @@ __global__ void __launch_bounds__(256, 2) attn_fwd_bf16(AttnParams p) {
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
+  // the forward keeps the tile-major order at every length: one slice after the other measures 2 % slower on 32 x 16384 rows
   if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -182,7 +183,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_q_bf16(AttnParams p) {
   constexpr int KK = D / 16, NC = D / 32, TILE = TS * 2 * D, STAGE = 2 * TILE;
 
   int bh, tile;
-  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, p.tile_major_q != 0, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -276,7 +277,7 @@ __global__ void __launch_bounds__(256, 2) attn_bwd_k_bf16(AttnParams p) {
   constexpr int STAGE = 2 * TILE + STAT;   // Q tile, dO tile, statistics
 
   int bh, tile;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, p.tile_major_k != 0, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;

@@ -686,7 +686,7 @@ __global__ void __launch_bounds__(PC_THREADS) attn_bwd_k_pc(AttnParams p) {
   constexpr int NC = D / 32;
 
   int bh, tile;
-  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, MASK != MASK_NONE, bh, tile)) return;
+  if (!decode_block((p.n_k + WG_ROWS - 1) / WG_ROWS, p.batch, false, p.tile_major_k != 0, bh, tile)) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool producer = wave < 4;

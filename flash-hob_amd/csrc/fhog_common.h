@@ -86,6 +86,8 @@ struct AttnParams {
   int32_t f16;       // tensors are fp16 (else bf16)
   int32_t mask_off;  // key j is visible to query i iff 0 <= i + mask_off - j < window
   int32_t window;
+  // Workgroup order within an XCD for the Q-tiled kernels (forward, dQ) and the K-tiled one (dK, dV): see Params
+  int32_t tile_major_q, tile_major_k;
 };
 
 // A kernel that uses more than 64 KiB of dynamic LDS needs its limit raised before the first launch. Done once per
