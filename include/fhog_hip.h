@@ -103,7 +103,7 @@ extern "C" {
  * list of key=value read once, on the host, at the first launch of the process (never in a timed path):
  *   b8=0|1            b and dd+b sweeps at d = 128: 128-row workgroups of 4 waves | 256-row workgroups of 8 waves
  *   order=slice|tile  workgroup order within an XCD: one (batch*head) slice after the other | the slices of an XCD advance
- *                     through their tiles together
+ *                     through their tiles together (also read by the first-order dQ and dK, dV kernels)
  *   split=0|1         small launches may split their streamed side over several workgroups (needs the workspace of
  *                     fhog_bwdbwd_workspace_hint)
  *   dd64=0|1          dd sweep at d = 128 with 32 | 64 queries per wave
