@@ -176,6 +176,8 @@ int run_pass(const fhog_bwdbwd_args* a, const fhog::Params& base, int impl, int 
   hipError_t e;
   if (pass > FHOG_PASS_DD_B && impl != FHOG_IMPL_BF16)
     return fail(FHOG_E_PASS, "pass %d exists in the 16-bit MFMA family only (bf16 / fp16 tensors, d in {64, 128})", pass);
+  if (pass == FHOG_PASS_STAGE1 && a->d != 64)
+    return fail(FHOG_E_PASS, "pass %d (three sweeps in one launch) exists for d = 64 only", pass);
   if (pass == FHOG_PASS_D)
     e = fhog::launch_rowdot(p, a->dtype, s);
   else if (impl == FHOG_IMPL_BF16)
@@ -304,6 +306,7 @@ const Tuning& tuning() {
       else if (!strcmp(tok, "split")) flag(tok, val, &r.split);
       else if (!strcmp(tok, "dd64")) flag(tok, val, &r.dd64);
       else if (!strcmp(tok, "stage64")) flag(tok, val, &r.stage64);
+      else if (!strcmp(tok, "stage1")) flag(tok, val, &r.stage1);
       else if (!strcmp(tok, "order")) {
         if (!strcmp(val, "tile")) r.order = 1;
         else if (!strcmp(val, "slice")) r.order = 0;
@@ -386,7 +389,7 @@ int fhog_select_impl(const fhog_bwdbwd_args* args) {
 int fhog_bwdbwd_pass(const fhog_bwdbwd_args* args, int pass, void* hip_stream) {
   const int rc = validate(args);
   if (rc != FHOG_OK) return rc;
-  if (pass < FHOG_PASS_D || pass > FHOG_PASS_DD_B_DDO) return fail(FHOG_E_PASS, "unknown pass %d", pass);
+  if (pass < FHOG_PASS_D || pass > FHOG_PASS_STAGE1) return fail(FHOG_E_PASS, "unknown pass %d", pass);
   const fhog::Params p = to_params(args);
   return run_pass(args, p, select_impl(args), pass, (hipStream_t)hip_stream);
 }
@@ -405,6 +408,11 @@ int fhog_bwdbwd(const fhog_bwdbwd_args* args, void* hip_stream) {
   static const int three[] = {FHOG_PASS_DD_B_DDO, FHOG_PASS_DQ, FHOG_PASS_DK_DV};
   const int* order = four;
   int first = impl == FHOG_IMPL_BF16 ? 1 : 0, n_pass = 5;
+  // d = 64, launch large enough to fill the GPU: the reference's own arrangement of its four passes, sweeps 1-3 in one launch
+  static const int stage1[] = {FHOG_PASS_STAGE1, FHOG_PASS_DK_DV};
+  if (args->schedule == FHOG_SCHEDULE_FOUR_PASS && impl == FHOG_IMPL_BF16 && args->d == 64 && fhog::tuning().stage1 != 0 &&
+      granted_split(args, impl, FHOG_PASS_DQ_DDO) == 1 && granted_split(args, impl, FHOG_PASS_DD) == 1)
+    order = stage1, first = 0, n_pass = 2;
   if (args->schedule == FHOG_SCHEDULE_FUSED_STATS) order = fused, n_pass = 4;
   // Passes 6-8 have no split form: a launch too small to fill the GPU whose workspace lets the reference's passes split
   // their streamed side runs the nearest schedule that can (three sweeps -> fused statistics, ddO early -> four passes).

@@ -66,11 +66,17 @@ __global__ void __launch_bounds__(256) combine_out(const float* part, int n_spli
   *reinterpret_cast<u32x2_t*>(out1 + o) = pack4<F16>(b[0], b[1], b[2], b[3]);
 }
 
-// SUB: 32-row tiles staged and consumed per barrier. SUB = 2 is a 64-row stage: one barrier, one round of staging
-// issues and one set of stage addresses per two blocks (twice the LDS), for the head dim whose blocks are short.
-template <bool F16, int D, int PASS, int MASK, int NW = 4, int SUB = 1>
-__global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+// Row statistics of the wave's queries handed from one sweep to the next inside a launch that runs several of them for
+// its tile (q_stage1_bf16): every lane of a query's pair holds the value.
+struct RowChain {
+  float d, dd, b;
+};
+
+// One Q-tiled sweep for the tile (bh, tile, split). CHAIN: the sweep is one of several that a launch runs for its tile;
+// it takes d, dd, b from `chain` where a sweep before it left them, and leaves there what it produces (it still writes
+// them to the workspace for the launches behind it).
+template <bool F16, int D, int PASS, int MASK, int NW, int SUB, bool CHAIN>
+__device__ __forceinline__ void q_sweep_run(const Params& p, char* smem, int bh, int tile, int split, RowChain& chain) {
   constexpr int ROWS = 32 * NW;
   constexpr int NT = (PASS == 1) ? 2 : 4;  // streamed tensors: K, ddK (, V, ddV)
   // PASS 7 is pass 3 without its ddO half (dQ2 alone, for the schedules whose earlier sweep already produced ddO)
@@ -79,10 +85,6 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   constexpr int STAGE = NT * TILE;
   constexpr int KK = D / 16;
 
-  // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
-  int bh, tile, split = 0;
-  if (!decode_block((p.n_q + ROWS - 1) / ROWS, p.batch * p.n_split, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
-  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: lets the compiler branch on scalars
   const int n = lane & 31, h = lane >> 5;
@@ -130,7 +132,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
   const float c_scale_log2 = p.scale * kLog2e;
   float dsum = 0.f;
   if (PASS == 2 || P3) {
-    dsum = p.ws_d[row];
+    dsum = CHAIN ? chain.d : p.ws_d[row];
   } else {
     // The first statistics sweep of a chain also produces d_i = sum_c O_ic dO_ic (fhog/triton_bwdbwd.py:580) for the
     // sweeps behind it: each lane holds half of its query's row of O and dO, one cross-half shuffle completes the sum.
@@ -143,9 +145,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(to_f32<F16>(Ob[kk][e]), to_f32<F16>(dOb[kk][e]), dsum);
     dsum += __shfl_xor(dsum, 32);
     if (h == 0 && qi < p.n_q && split == 0) p.ws_d[row] = dsum;
+    if (CHAIN) chain.d = dsum;
   }
-  const float dd = (PASS == 2 || P3) ? p.ws_dd[row] : 0.f;
-  const float b = P3 ? p.ws_b[row] : 0.f;
+  const float dd = (PASS == 2 || P3) ? (CHAIN ? chain.dd : p.ws_dd[row]) : 0.f;
+  const float b = P3 ? (CHAIN ? chain.b : p.ws_b[row]) : 0.f;
   const float kc = __builtin_fmaf(dd, dsum, b);   // per-row constant of dP' = E + (ddS - dd)(dP - d) - kc (passes 2, 3)
   float red = 0.f, red_dd = 0.f, red_pdp = 0.f;  // the last two: fused sweep only
   // PASS 3 (d = 64): the second-level products follow in the same wave, with the S-shaped tiles as B operands
@@ -407,9 +410,38 @@ __global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params 
       p.ws_dd[row] = dd_i;
       p.ws_b[row] = __builtin_fmaf(-dd_i, red_pdp, red);
     }
-  } else if (h == 0 && qi < p.n_q) {
-    (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
+  } else {
+    if (h == 0 && qi < p.n_q) (PASS == 1 ? p.ws_dd : p.ws_b)[row] = red;
+    if (CHAIN) (PASS == 1 ? chain.dd : chain.b) = red;
   }
+}
+
+// SUB: 32-row tiles staged and consumed per barrier. SUB = 2 is a 64-row stage: one barrier, one round of staging
+// issues and one set of stage addresses per two blocks (twice the LDS), for the head dim whose blocks are short.
+template <bool F16, int D, int PASS, int MASK, int NW = 4, int SUB = 1>
+__global__ void __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) q_sweep_bf16(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  // with a split, n_split consecutive "slices" share one (batch*head) slice and take its streamed tiles in turn
+  int bh, tile, split = 0;
+  if (!decode_block((p.n_q + 32 * NW - 1) / (32 * NW), p.batch * p.n_split, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
+  if (p.n_split > 1) split = bh % p.n_split, bh /= p.n_split;
+  RowChain unused;
+  q_sweep_run<F16, D, PASS, MASK, NW, SUB, false>(p, smem, bh, tile, split, unused);
+}
+
+// The reference's first kernel (bwdbwd_kernel_stage1, fhog/triton_bwdbwd.py:185-313) as it stands there: ONE launch
+// whose workgroups run the dd sweep, the b sweep and the dQ2 / ddO sweep one after the other for their query tile, dd
+// and b staying in registers in between. Same sweeps, same 25 products, two launches and two sets of resident loads
+// fewer. For the head dim whose three sweeps have the same workgroup shape (d = 64: 128 queries, four waves).
+template <bool F16, int D, int MASK>
+__global__ void __launch_bounds__(256, 2) q_stage1_bf16(Params p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int bh, tile;
+  if (!decode_block((p.n_q + WG_ROWS - 1) / WG_ROWS, p.batch, MASK != MASK_NONE, p.tile_major, bh, tile)) return;
+  RowChain chain;
+  q_sweep_run<F16, D, 1, MASK, 4, 1, true>(p, smem, bh, tile, 0, chain);   // every sweep ends on a barrier: the ring is free
+  q_sweep_run<F16, D, 2, MASK, 4, 1, true>(p, smem, bh, tile, 0, chain);
+  q_sweep_run<F16, D, 3, MASK, 4, 1, true>(p, smem, bh, tile, 0, chain);
 }
 
 // ---- pass 1 with 64 stationary rows per wave -----------------------------------------------------------------------
@@ -862,6 +894,14 @@ hipError_t launch_single_d(const Params& p, int pass, hipStream_t s) {
         return hipErrorInvalidValue;
       }
       break;
+    case FHOG_PASS_STAGE1:
+      if constexpr (D == 64) {
+        if (split) return hipErrorInvalidValue;
+        e = launch_sweep<q_stage1_bf16<F16, D, MASK>>(gq, 2 * 4 * tile, s, p);
+      } else {
+        return hipErrorInvalidValue;
+      }
+      break;
     case FHOG_PASS_DQ:
       if constexpr (D == 64) {
         e = two ? launch_sweep<q_sweep_bf16<F16, D, 7, MASK, 4, S2>>(gq, 2 * S2 * 4 * tile, s, p)
@@ -914,7 +954,7 @@ hipError_t launch_bf16_pass(const Params& p, int pass, hipStream_t s) {
     else hipLaunchKernelGGL((combine_out<false, 128>), grid, dim3(256), 0, s, p.part, p.n_split, p.batch, n, sb, sn, out0, out1, p.scale);
     return hipGetLastError();
   }
-  if (pass < FHOG_PASS_DD || pass > FHOG_PASS_DQ || pass == FHOG_PASS_B_DDO) return hipErrorInvalidValue;
+  if (pass != FHOG_PASS_STAGE1 && (pass < FHOG_PASS_DD || pass > FHOG_PASS_DQ || pass == FHOG_PASS_B_DDO)) return hipErrorInvalidValue;
   const int mask = mask_mode(p);
 #define FHOG_SINGLE(F, DD)                                                             \
   (mask == MASK_NONE ? launch_single_d<F, DD, MASK_NONE>(p, pass, s)                   \

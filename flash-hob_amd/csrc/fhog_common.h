@@ -62,8 +62,10 @@ struct Params {
 //   split=0|1          let launches too small to fill the GPU split their streamed side over several workgroups (default 1)
 //   dd64=0|1           dd sweep at d = 128: 32 | 64 queries per wave (default: 64 when that still gives 2048 workgroups)
 //   stage64=0|1        single-role sweeps at d = 64: one | two 32-row tiles staged and consumed per barrier (default 0: measured equal within 1 %)
+//   stage1=0|1         d = 64, reference schedule: sweeps 1-3 as three launches | as one launch whose workgroups run them one
+//                      after the other for their tile (FHOG_PASS_STAGE1)
 struct Tuning {
-  int b8 = -1, order = -1, split = 1, dd64 = -1, stage64 = 0;
+  int b8 = -1, order = -1, split = 1, dd64 = -1, stage64 = 0, stage1 = 0;
 };
 const Tuning& tuning();
 

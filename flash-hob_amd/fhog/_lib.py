@@ -15,7 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libfhog_hip.so"
 DTYPE_BF16, DTYPE_FP32, DTYPE_FP16 = 0, 1, 2
 IMPL_AUTO, IMPL_FP32, IMPL_BF16 = 0, 1, 2
 MASK_NONE, MASK_TOP_LEFT, MASK_BOTTOM_RIGHT = 0, 1, 2
-PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B, PASS_B_DDO, PASS_DQ, PASS_DD_B_DDO = range(9)
+PASS_D, PASS_DD, PASS_B, PASS_DQ_DDO, PASS_DK_DV, PASS_DD_B, PASS_B_DDO, PASS_DQ, PASS_DD_B_DDO, PASS_STAGE1 = range(10)
 SCHEDULE_FOUR_PASS, SCHEDULE_FUSED_STATS, SCHEDULE_DDO_EARLY, SCHEDULE_THREE_SWEEP = range(4)
 ABI_VERSION = 5
 STATIC_WS_BYTES = 16 << 20   # of a default build; `lib().fhog_static_ws_bytes()` tells what the loaded library holds

@@ -43,7 +43,7 @@ def pass_of(kernel):
         return 6 if m.group(1) == "true" else 8
     if re.match(r"q_sweep3_pc<\w+, \d+, \d, true>", kernel):
         return 7
-    for prefix, p in (("dd_sweep64_bf16", 1), ("q_sweep3_pc", 3), ("k_sweep_pc", 4), ("k_sweep_bf16", 4), ("rowdot", 0), ("attn_fwd", "fwd"),
+    for prefix, p in (("dd_sweep64_bf16", 1), ("q_stage1_bf16", 9), ("q_sweep3_pc", 3), ("k_sweep_pc", 4), ("k_sweep_bf16", 4), ("rowdot", 0), ("attn_fwd", "fwd"),
                       ("attn_bwd_q", "bwd_q"), ("attn_bwd_k", "bwd_k")):
         if kernel.startswith(prefix):
             return p
@@ -56,7 +56,7 @@ def algorithmic_mib(w, p):
     qt, kt, rv = w.batch * w.n_q * w.d * es / 2 ** 20, w.batch * w.n_k * w.d * es / 2 ** 20, w.batch * w.n_q * 4 / 2 ** 20
     table = {0: (2 * qt, rv), 1: (4 * qt + 2 * kt + rv, 2 * rv), 2: (3 * qt + 4 * kt + 3 * rv, rv),
              5: (4 * qt + 4 * kt + rv, 3 * rv), 6: (3 * qt + 4 * kt + 3 * rv, qt + rv), 7: (3 * qt + 4 * kt + 4 * rv, qt),
-             8: (4 * qt + 4 * kt + rv, qt + 3 * rv), 3: (3 * qt + 4 * kt + 4 * rv, 2 * qt), 4: (3 * qt + 4 * kt + 4 * rv, 2 * kt),
+             8: (4 * qt + 4 * kt + rv, qt + 3 * rv), 9: (4 * qt + 4 * kt + rv, 2 * qt + 3 * rv), 3: (3 * qt + 4 * kt + 4 * rv, 2 * qt), 4: (3 * qt + 4 * kt + 4 * rv, 2 * kt),
              "fwd": (qt + 2 * kt, qt + rv), "bwd_q": (2 * qt + 2 * kt + 2 * rv, qt), "bwd_k": (2 * qt + 2 * kt + 2 * rv, 2 * kt)}
     return table.get(p)
 

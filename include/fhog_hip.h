@@ -68,6 +68,10 @@ extern "C" {
 #define FHOG_PASS_DD_B_DDO 8 /* passes 1 and 6 in one sweep: dd_i is accumulated next to (P ddV)_i and ((P o ddS) V)_i
                                 and taken out at the end of the row, ddO_i = ... - dd_i O_i (sum_j P_ij V_j = O_i);
                                 writes d, dd, b, ddO */
+#define FHOG_PASS_STAGE1 9     /* passes 1, 2 and 3 in ONE launch whose workgroups run the three sweeps one after the other
+                                for their query tile, dd and b staying in registers: the reference's first kernel as it
+                                stands there (bwdbwd_kernel_stage1, fhog/triton_bwdbwd.py:185-313). 16-bit family, d = 64,
+                                streamed side not split; writes d, dd, b, dQ2, ddO */
 
 /* kernel families (fhog_bwdbwd_args.impl) */
 #define FHOG_IMPL_AUTO 0   /* 16-bit MFMA kernels for bf16/fp16 tensors when the shape allows, else the fp32-MFMA kernels */
@@ -108,6 +112,7 @@ extern "C" {
  *                     fhog_bwdbwd_workspace_hint)
  *   dd64=0|1          dd sweep at d = 128 with 32 | 64 queries per wave
  *   stage64=0|1       single-role sweeps at d = 64: one | two 32-row tiles staged and consumed per barrier
+ *   stage1=0|1        d = 64, four-pass schedule: sweeps 1-3 as three launches | as one launch (FHOG_PASS_STAGE1)
  * Results do not depend on any of them beyond fp32 summation order (split) - the others are bit-identical. Unknown keys
  * and values are reported on stderr and ignored. */
 typedef struct fhog_bwdbwd_args {

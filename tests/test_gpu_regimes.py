@@ -104,9 +104,10 @@ torch.save(out, sys.argv[1])
 """
 # small, ragged and masked, d = 128: the 8-wave b and ddO sweeps, the 64-queries-per-wave dd sweep and both workgroup orders on
 # launches of a handful of workgroups (each case under the default and under the three-sweep schedule); the last shape is
-# one whose passes split their streamed side by default
+# one whose passes split their streamed side by default; d64_many: d = 64 with workgroups enough not to split (the one-launch
+# form of sweeps 1-3 and the 64-row stage apply)
 _TUNE_CASES = {"ragged_causal": ((3, 333, 333, 128), True, None), "window": ((2, 300, 400, 128), "bottom_right", 200),
-               "split": ((2, 700, 700, 128), True, None)}
+               "d64_many": ((180, 384, 300, 64), False, None), "split": ((2, 700, 700, 128), True, None)}
 
 
 def _run_child(tmp_path, tune):
@@ -119,10 +120,11 @@ def _run_child(tmp_path, tune):
 
 
 def test_launch_choices_forced_through_FHOG_TUNE(tmp_path):
-    """b8, dd64 and order change which kernel or which workgroup order runs, never a bit of the results; split=0 changes
-    the fp32 summation order of the launches that would split. Unknown keys are reported, not obeyed."""
+    """b8, dd64, order, stage64 and stage1 change which kernel, which workgroup order or how many launches run, never a bit
+    of the results; split=0 changes the fp32 summation order of the launches that would split. Unknown keys are reported,
+    not obeyed."""
     base, _ = _run_child(tmp_path, "")
-    for tune in ("b8=1,dd64=1,order=slice", "b8=0,dd64=0,order=tile"):
+    for tune in ("b8=1,dd64=1,order=slice,stage1=1", "b8=0,dd64=0,order=tile,stage64=1"):
         got, err = _run_child(tmp_path, tune)
         assert "FHOG_TUNE" not in err, err
         for tag in base:

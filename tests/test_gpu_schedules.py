@@ -105,10 +105,40 @@ def test_new_passes_exist_in_the_16_bit_family_only():
     x = with_caches(make_case(2, 128, 128, 64, torch.bfloat16, seed=56), 0.125, False)
     plan = BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125, impl="fp32")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for pass_id in (_lib.PASS_B_DDO, _lib.PASS_DQ, _lib.PASS_DD_B_DDO):
+    for pass_id in (_lib.PASS_B_DDO, _lib.PASS_DQ, _lib.PASS_DD_B_DDO, _lib.PASS_STAGE1):
         assert plan.lib.fhog_bwdbwd_pass(ctypes.byref(plan.args), pass_id, stream) == -7
         assert "16-bit" in plan.lib.fhog_last_error().decode()
-    assert plan.lib.fhog_bwdbwd_pass(ctypes.byref(plan.args), 9, stream) == -7
+    assert plan.lib.fhog_bwdbwd_pass(ctypes.byref(plan.args), 10, stream) == -7
+    # the one-launch form of sweeps 1-3 exists where the three sweeps share a workgroup shape: d = 64
+    y = with_caches(make_case(2, 128, 128, 128, torch.bfloat16, seed=56), 128 ** -0.5, False)
+    plan = BwdBwdPlan(y["Q"], y["K"], y["V"], y["O"], y["dO"], y["ddQ"], y["ddK"], y["ddV"], y["L"], 128 ** -0.5)
+    assert plan.lib.fhog_bwdbwd_pass(ctypes.byref(plan.args), _lib.PASS_STAGE1, stream) == -7
+    assert "d = 64" in plan.lib.fhog_last_error().decode()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", [(5, 640, 640, True, None), (3, 300, 777, "bottom_right", 200), (70, 256, 1000, False, None),
+                                  (2, 33, 129, False, None)])
+def test_three_sweeps_in_one_launch_equal_the_three_launches(case, dtype):
+    """FHOG_PASS_STAGE1, the reference's own arrangement (bwdbwd_kernel_stage1 runs its three sweeps inside one kernel,
+    fhog/triton_bwdbwd.py:185-313): same sweeps with dd and b handed over in registers, so d, dd, b, dQ2 and ddO come out
+    bit for bit as from passes 1, 2, 3 launched one by one."""
+    from fhog import BwdBwdPlan, _lib
+    batch, n_q, n_k, causal, window = case
+    x = with_caches(make_case(batch, n_q, n_k, 64, dtype, seed=61, grad_std=0.1), 0.125, causal, window)
+    plans = [BwdBwdPlan(x["Q"], x["K"], x["V"], x["O"], x["dO"], x["ddQ"], x["ddK"], x["ddV"], x["L"], 0.125, causal=causal,
+                        window=window, split=False) for _ in range(2)]
+    for p in plans:
+        for t in p.outs:
+            t.fill_(float("nan"))
+        p.ws.fill_(float("nan"))
+    for pass_id in (_lib.PASS_DD, _lib.PASS_B, _lib.PASS_DQ_DDO):
+        plans[0].run(only_pass=pass_id)
+    plans[1].run(only_pass=_lib.PASS_STAGE1)
+    torch.cuda.synchronize()
+    assert torch.equal(plans[0].ws, plans[1].ws) and torch.isfinite(plans[0].ws).all()
+    for a, b in ((plans[0].outs[0], plans[1].outs[0]), (plans[0].outs[3], plans[1].outs[3])):   # dQ2, ddO
+        assert torch.equal(a, b) and torch.isfinite(a.float()).all()
 
 
 def _full_config(name, seed, schedule, heads=None):
