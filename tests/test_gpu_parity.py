@@ -285,7 +285,10 @@ def test_split_streamed_side_matches_the_unsplit_launch(case, fused_stats):
     """Few (batch*head) slices: with the workspace of fhog_bwdbwd_workspace_hint every pass splits its
     streamed side over several workgroups (fp32 partial results, added by a second kernel). Same gate against the
     fp64 oracle as the unsplit launch, row statistics equal up to summation order, outputs within a 16-bit rounding."""
+    import os
     from fhog import BwdBwdPlan, _lib
+    if "split=0" in os.environ.get("FHOG_TUNE", ""):
+        pytest.skip("FHOG_TUNE switches the split launches off")
     (batch, n_q, n_k, d), causal, window, dtype = case
     scale = d ** -0.5
     x = with_caches(make_case(batch, n_q, n_k, d, dtype, seed=23, grad_std=0.1), scale, causal, window)
